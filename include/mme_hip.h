@@ -200,6 +200,24 @@ int mme_hip_set_stream(mme_hip_handle h, void* hip_stream);
 /* hipStreamSynchronize on the handle's stream. */
 int mme_hip_synchronize(mme_hip_handle h);
 
+/*
+ * fp8 operands and the matrix cores.  gfx950's MFMA reads OCP e4m3 / e5m2.  Gaudi's fp8_152 in full inf/nan mode is
+ * e5m2 up to the exponent bias, and fp8_143 in minimal inf/nan mode is e4m3; the bias becomes an exact power of two
+ * on the accumulators.  In the other modes the codes with all exponent bits set mean something else to the hardware
+ * (fp8_143 full mode: inf / NaN, fs_fma.cpp:6090-6100, but 256..448 for e4m3).
+ *   MME_HIP_FP8_SPECIALS_CHECK (default): operands in such modes are scanned on the device; if a scan finds such a
+ *     code the contraction runs on an exact bf16 decode of both operands instead.  No host synchronisation.
+ *   MME_HIP_FP8_SPECIALS_ASSUME_NONE: the caller guarantees there are none (e.g. the operands come out of a
+ *     saturating quantiser, which never emits them); the scan is skipped.
+ * No counterpart in the reference, which decodes every element in software.
+ */
+enum
+{
+    MME_HIP_FP8_SPECIALS_CHECK = 0,
+    MME_HIP_FP8_SPECIALS_ASSUME_NONE = 1
+};
+int mme_hip_set_fp8_specials_policy(mme_hip_handle h, int policy);
+
 /* ---- contraction: host pointers (reference-compatible, synchronous) ------ */
 
 /*

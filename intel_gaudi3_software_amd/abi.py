@@ -25,6 +25,7 @@ OP_FWD, OP_DEDX, OP_DEDW, OP_DETERMINISTIC_DEDW, OP_TRANSPOSED_DEDX, OP_AB, OP_A
 # InfNanMode
 FULL_INF_NAN, NO_INF_NAN, MINIMAL_INF_NAN = 0, 1, 2
 REDUCTION_NONE = 0
+FP8_SPECIALS_CHECK, FP8_SPECIALS_ASSUME_NONE = 0, 1
 
 DTYPE_SIZE = {FP8_143: 1, FP8_152: 1, FP16: 2, BF16: 2, FP32: 4, FP32_IEEE: 4, TF32: 4}
 DTYPE_NUMPY = {FP8_143: np.uint8, FP8_152: np.uint8, BF16: np.uint16, FP16: np.uint16, FP32: np.float32,
@@ -135,13 +136,14 @@ def load_library():
     L.mme_hip_stream.restype = vp
     L.mme_hip_set_stream.argtypes = [vp, vp]
     L.mme_hip_synchronize.argtypes = [vp]
+    L.mme_hip_set_fp8_specials_policy.argtypes = [vp, C.c_int]
     L.mme_hip_batch_gemm.argtypes = [vp, _TP, _TP, _TP, C.c_int, C.c_int, C.c_int, C.c_int]
     L.mme_hip_convolution.argtypes = [vp, _TP, _TP, _TP, _TP, C.POINTER(ConvParams), C.c_int, C.c_int, C.c_int, C.c_int]
-    L.mme_hip_activation.argtypes = [vp, _TP, _TP] + [C.c_int] * 7
+    L.mme_hip_activation.argtypes = [vp, _TP, _TP] + [C.c_int] * 6
     L.mme_hip_memory_write.argtypes = [vp, _TP, _TP, C.c_int, C.c_int, C.c_int]
     L.mme_hip_batch_gemm_dev.argtypes = [vp, _TP, _TP, _TP, C.c_int, C.POINTER(Epilogue)]
     L.mme_hip_convolution_dev.argtypes = [vp, _TP, _TP, _TP, _TP, C.POINTER(ConvParams), C.c_int, C.POINTER(Epilogue)]
-    L.mme_hip_activation_dev.argtypes = [vp, _TP, _TP] + [C.c_int] * 7
+    L.mme_hip_activation_dev.argtypes = [vp, _TP, _TP] + [C.c_int] * 6
     L.mme_hip_cast_from_fp32_dev.argtypes = [vp, vp, C.c_int, C.c_uint, C.c_int, vp, C.c_size_t, C.c_int, vp,
                                              C.c_size_t] + [C.c_int] * 5
     L.mme_hip_cast_to_fp32_dev.argtypes = [vp, vp, vp, C.c_int, C.c_uint, C.c_int, C.c_size_t, C.c_int, vp, C.c_size_t]

@@ -1,0 +1,393 @@
+// cast_kernels.hip -- bandwidth-bound elementwise kernels: fp32 -> {fp8_143, fp8_152, bf16, fp32} (cast / quantize),
+// {fp8, bf16} -> fp32 (dequantize), in-place relu, absmax.
+//
+// Each follows convertToOutputDataType (mme/mme_reference/mme_reference_impl.cpp:1143-1245) element by element; the
+// arithmetic lives in mme_numeric.hpp.  Layout: flat arrays.  A wavefront reads 64 x 16 B = 1 KiB per load
+// instruction (fully coalesced) and keeps four such loads in flight per lane; algorithmic traffic is 4 + sizeof(out)
+// bytes per element (5 B for fp8, 6 B for bf16), the kernels are HBM-bound.
+#include "mme_kernels.hpp"
+
+namespace mme
+{
+namespace
+{
+typedef float    v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+
+constexpr int CAST_THREADS = 256;
+constexpr int CAST_UNROLL = 4; // float4 loads in flight per lane
+
+template<int DT>
+struct OutVec; // four converted elements
+template<>
+struct OutVec<DT_FP8_143>
+{
+    using type = uint32_t;
+};
+template<>
+struct OutVec<DT_FP8_152>
+{
+    using type = uint32_t;
+};
+template<>
+struct OutVec<DT_BF16>
+{
+    using type = v2u;
+};
+template<>
+struct OutVec<DT_FP32>
+{
+    using type = v4u;
+};
+
+// the per-tensor power of two; skipped (not multiplied by 1) when absent so that NaN payloads reach an fp32 output intact
+__device__ __forceinline__ float descale(float v, const CastParams& p) { return p.has_scale ? v * p.scale : v; }
+
+template<int DT, bool FAST>
+__device__ __forceinline__ typename OutVec<DT>::type cast4(const v4f& v, const CastParams& p, const v4f& cs)
+{
+    const uint32_t a = cast_elem<DT, FAST>(descale(v.x, p) * cs.x, p), b = cast_elem<DT, FAST>(descale(v.y, p) * cs.y, p),
+                   c = cast_elem<DT, FAST>(descale(v.z, p) * cs.z, p), d = cast_elem<DT, FAST>(descale(v.w, p) * cs.w, p);
+    if constexpr (DT == DT_FP8_143 || DT == DT_FP8_152) return a | (b << 8) | (c << 16) | (d << 24);
+    else if constexpr (DT == DT_BF16)
+        return v2u {a | (b << 16), c | (d << 16)};
+    else
+        return v4u {a, b, c, d};
+}
+template<int DT, bool FAST>
+__device__ __forceinline__ typename OutVec<DT>::type cast4(const v4f& v, const CastParams& p)
+{
+    const uint32_t a = cast_elem<DT, FAST>(descale(v.x, p), p), b = cast_elem<DT, FAST>(descale(v.y, p), p),
+                   c = cast_elem<DT, FAST>(descale(v.z, p), p), d = cast_elem<DT, FAST>(descale(v.w, p), p);
+    if constexpr (DT == DT_FP8_143 || DT == DT_FP8_152) return a | (b << 8) | (c << 16) | (d << 24);
+    else if constexpr (DT == DT_BF16)
+        return v2u {a | (b << 16), c | (d << 16)};
+    else
+        return v4u {a, b, c, d};
+}
+
+template<int DT>
+__device__ __forceinline__ void store1(void* out, size_t i, uint32_t v)
+{
+    if constexpr (DT == DT_FP8_143 || DT == DT_FP8_152) ((uint8_t*) out)[i] = (uint8_t) v;
+    else if constexpr (DT == DT_BF16)
+        ((uint16_t*) out)[i] = (uint16_t) v;
+    else
+        ((uint32_t*) out)[i] = v;
+}
+
+__device__ __forceinline__ float pow2_of(int e) { return u2f((uint32_t) (e + 127) << 23); }
+
+// n4 = number of whole float4 groups; the tail (n % 4 elements) is handled by the last lanes of block 0.
+// COL: multiply element i by 2^col_exp[i % n_cols] as well (n_cols % 4 == 0 is required by the launcher for COL).
+template<int DT, bool FAST, bool COL>
+__global__ __launch_bounds__(CAST_THREADS) void cast_from_fp32_kernel(void* __restrict__ out,
+                                                                      const float* __restrict__ in,
+                                                                      size_t n,
+                                                                      CastParams p,
+                                                                      const int32_t* __restrict__ col_exp,
+                                                                      uint32_t n_cols)
+{
+    using OV = typename OutVec<DT>::type;
+    const size_t  n4 = n >> 2;
+    const v4f*    in4 = reinterpret_cast<const v4f*>(in);
+    OV*           out4 = reinterpret_cast<OV*>(out);
+    const size_t  stride = (size_t) gridDim.x * CAST_THREADS;
+    size_t        i = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x;
+
+    for (; i + (CAST_UNROLL - 1) * stride < n4; i += CAST_UNROLL * stride)
+    {
+        v4f v[CAST_UNROLL];
+#pragma unroll
+        for (int j = 0; j < CAST_UNROLL; j++) v[j] = __builtin_nontemporal_load(in4 + i + j * stride);
+#pragma unroll
+        for (int j = 0; j < CAST_UNROLL; j++)
+        {
+            OV o;
+            if constexpr (COL)
+            {
+                const uint32_t c0 = (uint32_t) (((i + j * stride) << 2) % n_cols);
+                const int4     ce = *reinterpret_cast<const int4*>(col_exp + c0);
+                o = cast4<DT, FAST>(v[j], p, v4f {pow2_of(ce.x), pow2_of(ce.y), pow2_of(ce.z), pow2_of(ce.w)});
+            }
+            else
+                o = cast4<DT, FAST>(v[j], p);
+            __builtin_nontemporal_store(o, out4 + i + j * stride);
+        }
+    }
+    for (; i < n4; i += stride)
+    {
+        const v4f v = in4[i];
+        OV        o;
+        if constexpr (COL)
+        {
+            const uint32_t c0 = (uint32_t) ((i << 2) % n_cols);
+            const int4     ce = *reinterpret_cast<const int4*>(col_exp + c0);
+            o = cast4<DT, FAST>(v, p, v4f {pow2_of(ce.x), pow2_of(ce.y), pow2_of(ce.z), pow2_of(ce.w)});
+        }
+        else
+            o = cast4<DT, FAST>(v, p);
+        out4[i] = o;
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 3))
+    {
+        const size_t k = (n4 << 2) + threadIdx.x;
+        float        v = in[k];
+        if (p.has_scale) v *= p.scale;
+        if constexpr (COL) v *= pow2_of(col_exp[k % n_cols]);
+        store1<DT>(out, k, cast_elem<DT, FAST>(v, p));
+    }
+}
+
+// scalar form for per-column scales whose period is not a multiple of 4, or unaligned buffers
+template<int DT, bool FAST>
+__global__ __launch_bounds__(CAST_THREADS) void cast_from_fp32_scalar_kernel(void* __restrict__ out,
+                                                                             const float* __restrict__ in,
+                                                                             size_t n,
+                                                                             CastParams p,
+                                                                             const int32_t* __restrict__ col_exp,
+                                                                             uint32_t n_cols)
+{
+    const size_t stride = (size_t) gridDim.x * CAST_THREADS;
+    for (size_t i = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x; i < n; i += stride)
+    {
+        float v = in[i];
+        if (p.has_scale) v *= p.scale;
+        if (col_exp) v *= pow2_of(col_exp[i % n_cols]);
+        store1<DT>(out, i, cast_elem<DT, FAST>(v, p));
+    }
+}
+
+// ---- dequantize -----------------------------------------------------------------------------------------------
+template<int DT>
+__device__ __forceinline__ float decode1(uint32_t code, int bias, int mode)
+{
+    if constexpr (DT == DT_FP8_143) return u2f(fp8_to_fp32<3>(code, bias, mode));
+    else if constexpr (DT == DT_FP8_152)
+        return u2f(fp8_to_fp32<2>(code, bias, mode));
+    else
+        return u2f(code << 16);
+}
+
+template<int DT>
+__global__ __launch_bounds__(CAST_THREADS) void cast_to_fp32_kernel(float* __restrict__ out,
+                                                                    const void* __restrict__ in,
+                                                                    size_t n,
+                                                                    int bias,
+                                                                    int mode,
+                                                                    float scale,
+                                                                    int has_scale,
+                                                                    const int32_t* __restrict__ col_exp,
+                                                                    uint32_t n_cols,
+                                                                    int vec_ok)
+{
+    const size_t stride = (size_t) gridDim.x * CAST_THREADS;
+    const size_t t = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x;
+    size_t       done = 0;
+    if (vec_ok)
+    {
+        // four elements per lane and step: one 4 B (fp8) / 8 B (bf16) load, one 16 B store
+        const size_t n4 = n >> 2;
+        float4*      out4 = reinterpret_cast<float4*>(out);
+        for (size_t i = t; i < n4; i += stride)
+        {
+            uint32_t c[4];
+            if constexpr (DT == DT_BF16)
+            {
+                const uint2 r = reinterpret_cast<const uint2*>(in)[i];
+                c[0] = r.x & 0xFFFFu;
+                c[1] = r.x >> 16;
+                c[2] = r.y & 0xFFFFu;
+                c[3] = r.y >> 16;
+            }
+            else
+            {
+                const uint32_t r = reinterpret_cast<const uint32_t*>(in)[i];
+                c[0] = r & 0xFFu;
+                c[1] = (r >> 8) & 0xFFu;
+                c[2] = (r >> 16) & 0xFFu;
+                c[3] = r >> 24;
+            }
+            float f[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+            {
+                f[j] = decode1<DT>(c[j], bias, mode);
+                if (has_scale) f[j] *= scale;
+                if (col_exp) f[j] *= pow2_of(col_exp[((i << 2) + j) % n_cols]);
+            }
+            out4[i] = make_float4(f[0], f[1], f[2], f[3]);
+        }
+        done = n4 << 2;
+    }
+    for (size_t i = done + t; i < n; i += stride)
+    {
+        uint32_t c;
+        if constexpr (DT == DT_BF16) c = reinterpret_cast<const uint16_t*>(in)[i];
+        else
+            c = reinterpret_cast<const uint8_t*>(in)[i];
+        float f = decode1<DT>(c, bias, mode);
+        if (has_scale) f *= scale;
+        if (col_exp) f *= pow2_of(col_exp[i % n_cols]);
+        out[i] = f;
+    }
+}
+
+__global__ __launch_bounds__(CAST_THREADS) void relu_inplace_kernel(float* __restrict__ x, size_t n)
+{
+    const size_t stride = (size_t) gridDim.x * CAST_THREADS;
+    for (size_t i = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x; i < n; i += stride) x[i] = relu_ref(x[i]);
+}
+
+// ---- absmax: wavefront reduction with DPP-free shuffles, one atomicMax on the bit pattern per block -------------
+__global__ __launch_bounds__(CAST_THREADS) void absmax_kernel(uint32_t* __restrict__ out_bits,
+                                                              const float* __restrict__ in,
+                                                              size_t n,
+                                                              int vec_ok)
+{
+    const size_t stride = (size_t) gridDim.x * CAST_THREADS;
+    const size_t t = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x;
+    uint32_t     m = 0; // |x| of non-NaN fp32 values orders like the unsigned bit pattern
+    auto         acc = [&](float f) {
+        const uint32_t a = f2u(f) & 0x7FFFFFFFu;
+        if (a <= 0x7F800000u) m = max(m, a);
+    };
+    size_t done = 0;
+    if (vec_ok)
+    {
+        const size_t  n4 = n >> 2;
+        const v4f*    in4 = reinterpret_cast<const v4f*>(in);
+        for (size_t i = t; i < n4; i += stride)
+        {
+            const v4f v = __builtin_nontemporal_load(in4 + i);
+            acc(v.x);
+            acc(v.y);
+            acc(v.z);
+            acc(v.w);
+        }
+        done = n4 << 2;
+    }
+    for (size_t i = done + t; i < n; i += stride) acc(in[i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t) __shfl_xor((int) m, off, 64));
+    __shared__ uint32_t wave_max[CAST_THREADS / 64];
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0)
+    {
+        uint32_t b = wave_max[0];
+        for (int w = 1; w < CAST_THREADS / 64; w++) b = max(b, wave_max[w]);
+        atomicMax(out_bits, b);
+    }
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, size_t n)
+{
+    const size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+int grid_for(size_t work_items, int max_blocks)
+{
+    size_t b = (work_items + CAST_THREADS - 1) / CAST_THREADS;
+    if (b < 1) b = 1;
+    if (b > (size_t) max_blocks) b = (size_t) max_blocks;
+    return (int) b;
+}
+
+template<int DT, bool FAST>
+void launch_cast_dt(void* out, const float* in, size_t n, const CastParams& p, const int32_t* col, size_t n_cols,
+                    hipStream_t s)
+{
+    const bool aligned = (((uintptr_t) out | (uintptr_t) in) & 15u) == 0;
+    // 2048 blocks x 256 lanes x 4 float4 = 32 MiB of input in flight per sweep: >> 256 CUs, few tail effects
+    if (aligned && (!col || ((n_cols & 3u) == 0 && ((uintptr_t) col & 15u) == 0)))
+    {
+        const int grid = grid_for((n >> 2) / CAST_UNROLL + 1, 4096);
+        if (col)
+            hipLaunchKernelGGL((cast_from_fp32_kernel<DT, FAST, true>), dim3(grid), dim3(CAST_THREADS), 0, s, out, in, n, p,
+                               col, (uint32_t) n_cols);
+        else
+            hipLaunchKernelGGL((cast_from_fp32_kernel<DT, FAST, false>), dim3(grid), dim3(CAST_THREADS), 0, s, out, in, n,
+                               p, col, (uint32_t) n_cols);
+    }
+    else
+    {
+        const int grid = grid_for(n, 8192);
+        hipLaunchKernelGGL((cast_from_fp32_scalar_kernel<DT, FAST>), dim3(grid), dim3(CAST_THREADS), 0, s, out, in, n, p,
+                           col, (uint32_t) (n_cols ? n_cols : 1));
+    }
+}
+} // namespace
+
+hipError_t launch_cast_from_fp32(void* out, const float* in, size_t n, const CastParams& p, const int32_t* col,
+                                 size_t n_cols, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    const bool fast = cast_params_fast(p);
+    switch (p.dtype)
+    {
+        case DT_FP8_143:
+            fast ? launch_cast_dt<DT_FP8_143, true>(out, in, n, p, col, n_cols, s)
+                 : launch_cast_dt<DT_FP8_143, false>(out, in, n, p, col, n_cols, s);
+            break;
+        case DT_FP8_152:
+            fast ? launch_cast_dt<DT_FP8_152, true>(out, in, n, p, col, n_cols, s)
+                 : launch_cast_dt<DT_FP8_152, false>(out, in, n, p, col, n_cols, s);
+            break;
+        case DT_BF16:
+            fast ? launch_cast_dt<DT_BF16, true>(out, in, n, p, col, n_cols, s)
+                 : launch_cast_dt<DT_BF16, false>(out, in, n, p, col, n_cols, s);
+            break;
+        case DT_FP32: launch_cast_dt<DT_FP32, false>(out, in, n, p, col, n_cols, s); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_cast_to_fp32(float* out, const void* in, int dtype, int bias, int mode, size_t n, float scale,
+                               int has_scale, const int32_t* col, size_t n_cols, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    const int vec_ok = (((uintptr_t) out & 15u) == 0) && (((uintptr_t) in & 7u) == 0);
+    const int grid = grid_for(vec_ok ? (n >> 2) + 1 : n, 8192);
+    const uint32_t nc = (uint32_t) (n_cols ? n_cols : 1);
+    switch (dtype)
+    {
+        case DT_FP8_143:
+            hipLaunchKernelGGL((cast_to_fp32_kernel<DT_FP8_143>), dim3(grid), dim3(CAST_THREADS), 0, s, out, in, n, bias,
+                               mode, scale, has_scale, col, nc, vec_ok);
+            break;
+        case DT_FP8_152:
+            hipLaunchKernelGGL((cast_to_fp32_kernel<DT_FP8_152>), dim3(grid), dim3(CAST_THREADS), 0, s, out, in, n, bias,
+                               mode, scale, has_scale, col, nc, vec_ok);
+            break;
+        case DT_BF16:
+            hipLaunchKernelGGL((cast_to_fp32_kernel<DT_BF16>), dim3(grid), dim3(CAST_THREADS), 0, s, out, in, n, bias, mode,
+                               scale, has_scale, col, nc, vec_ok);
+            break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s)
+{
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(relu_inplace_kernel, dim3(grid_for(n, 8192)), dim3(CAST_THREADS), 0, s, x, n);
+    return hipGetLastError();
+}
+
+hipError_t launch_absmax(float* out, const float* in, size_t n, hipStream_t s)
+{
+    // the result cell is cleared by a one-lane fill kernel (not a memset node) so the sequence can be graph-captured
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(1), 0, s, (uint32_t*) out, 0u, (size_t) 1);
+    if (n == 0) return hipGetLastError();
+    const int vec_ok = ((uintptr_t) in & 15u) == 0;
+    hipLaunchKernelGGL(absmax_kernel, dim3(grid_for(vec_ok ? (n >> 2) + 1 : n, 2048)), dim3(CAST_THREADS), 0, s,
+                       (uint32_t*) out, in, n, vec_ok);
+    return hipGetLastError();
+}
+
+} // namespace mme

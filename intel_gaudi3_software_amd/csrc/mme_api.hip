@@ -1,0 +1,808 @@
+// mme_api.hip -- the C ABI declared in include/mme_hip.h: handle, validation (the reference's MME_ASSERT conditions),
+// mapping of tensor descriptors to kernel problems, host-pointer staging.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "../../include/mme_hip.h"
+#include "mme_kernels.hpp"
+
+using namespace mme;
+
+namespace
+{
+thread_local std::string g_create_error = "";
+
+struct DeviceBuffer
+{
+    void*  p = nullptr;
+    size_t bytes = 0;
+    ~DeviceBuffer()
+    {
+        if (p) (void) hipFree(p);
+    }
+    hipError_t reserve(size_t n)
+    {
+        if (n <= bytes) return hipSuccess;
+        if (p) (void) hipFree(p);
+        p = nullptr;
+        bytes = 0;
+        hipError_t e = hipMalloc(&p, n);
+        if (e == hipSuccess) bytes = n;
+        return e;
+    }
+};
+} // namespace
+
+struct mme_hip_calc
+{
+    int                   chip = MME_HIP_CHIP_GAUDI3;
+    int                   device = 0;
+    int                   num_cus = 256;
+    hipStream_t           own_stream = nullptr;
+    hipStream_t           stream = nullptr;
+    unsigned              num_threads = 1;
+    std::vector<uint32_t> lfsr;
+    uint32_t              polynomial = 0;
+    std::string           error;
+    DeviceBuffer          split_ws;  // split-k partial sums
+    DeviceBuffer          decode_ws; // bf16 copies of fp8 operands the hardware formats cannot express
+    DeviceBuffer          flag;      // one 32-bit cell: "operands hold codes the hardware formats lack"
+    int                   fp8_specials_policy = 0;
+};
+
+namespace
+{
+int fail(mme_hip_handle h, int code, const char* fmt, ...)
+{
+    char    buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (h) h->error = buf;
+    else
+        g_create_error = buf;
+    return code;
+}
+
+int hip_fail(mme_hip_handle h, hipError_t e, const char* what)
+{
+    return fail(h, e == hipErrorOutOfMemory ? MME_HIP_ENOMEM : MME_HIP_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(h, expr)                                          \
+    do                                                            \
+    {                                                             \
+        hipError_t e_ = (expr);                                   \
+        if (e_ != hipSuccess) return hip_fail((h), e_, #expr);    \
+    } while (0)
+
+int elem_size(int dt)
+{
+    switch (dt)
+    {
+        case MME_HIP_FP8_143:
+        case MME_HIP_FP8_152: return 1;
+        case MME_HIP_BF16:
+        case MME_HIP_FP16: return 2;
+        case MME_HIP_FP32:
+        case MME_HIP_FP32_IEEE:
+        case MME_HIP_TF32: return 4;
+        default: return 0;
+    }
+}
+bool is_fp8(int dt) { return dt == MME_HIP_FP8_143 || dt == MME_HIP_FP8_152; }
+
+uint64_t n_elements(const mme_hip_tensor* t)
+{
+    uint64_t n = 1;
+    for (int d = 0; d < 5; d++) n *= t->sizes[d];
+    return n;
+}
+// elements spanned in memory: the largest stride * size (setStridesAndGetTensorSize, sim_tensor_base.cpp:351-374)
+uint64_t span_elements(const mme_hip_tensor* t)
+{
+    uint64_t m = 0;
+    for (int d = 0; d < 5; d++) m = std::max<uint64_t>(m, (uint64_t) t->strides[d] * t->sizes[d]);
+    return m;
+}
+// dims 1..4 enumerate rows of one dense-pitched matrix: stride[d+1] == stride[d] * size[d]
+bool rows_collapsible(const mme_hip_tensor* t)
+{
+    for (int d = 1; d < 4; d++)
+        if (t->sizes[d + 1] > 1 && (uint64_t) t->strides[d + 1] != (uint64_t) t->strides[d] * t->sizes[d]) return false;
+    return true;
+}
+
+int check_tensor(mme_hip_handle h, const mme_hip_tensor* t, const char* name)
+{
+    if (!t) return fail(h, MME_HIP_EINVAL, "%s: got null pointer", name);
+    if (elem_size(t->dtype) == 0) return fail(h, MME_HIP_EINVAL, "%s: type not supported", name);
+    if (t->dtype == MME_HIP_FP16 || t->dtype == MME_HIP_TF32)
+        return fail(h, MME_HIP_EUNSUPPORTED, "%s: fp16 / tf32 operands are not built in this library", name);
+    if (t->strides[0] != 1) return fail(h, MME_HIP_EINVAL, "%s: the first dimension must be contiguous", name);
+    if (n_elements(t) >= (1ull << 31)) return fail(h, MME_HIP_EINVAL, "%s: more than 2^31 elements", name);
+    if (n_elements(t) && !t->data) return fail(h, MME_HIP_EINVAL, "%s: got null pointer", name);
+    return MME_HIP_OK;
+}
+
+// the reference's registration table for Gaudi3 (mme_reference_impl.cpp:188-196) and its type pairing rule
+// (chip_fma/gaudi3_fma.cpp:62-66)
+int check_operand_types(mme_hip_handle h, const mme_hip_tensor* a, const mme_hip_tensor* b)
+{
+    const int ta = a->dtype, tb = b->dtype;
+    if (!(ta == MME_HIP_BF16 || ta == MME_HIP_FP32 || is_fp8(ta))) return fail(h, MME_HIP_EINVAL, "type is not registered in function map !");
+    if (!(is_fp8(ta) && is_fp8(tb)) && ta != tb) return fail(h, MME_HIP_EINVAL, "Gaudi3 doesnt support mixed input type flavors");
+    for (const mme_hip_tensor* t : {a, b})
+        if (is_fp8(t->dtype))
+        {
+            if (t->dtype == MME_HIP_FP8_143 && !(t->fp_bias == 3 || t->fp_bias == 7 || t->fp_bias == 11 || t->fp_bias == 15))
+                return fail(h, MME_HIP_EINVAL, "fp8_143 exponent bias must be 3, 7, 11 or 15");
+            if (t->dtype == MME_HIP_FP8_152 && (t->fp_bias < 1 || t->fp_bias > 30))
+                return fail(h, MME_HIP_EINVAL, "fp8_152 exponent bias must be in 1..30");
+            if (t->inf_nan_mode < 0 || t->inf_nan_mode > 2) return fail(h, MME_HIP_EINVAL, "invalid infNanMode");
+        }
+    return MME_HIP_OK;
+}
+
+int check_out_type(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_epilogue* epi)
+{
+    if (!epi)
+    {
+        if (out->dtype != MME_HIP_FP32) return fail(h, MME_HIP_EINVAL, "type is not registered in function map !");
+        return MME_HIP_OK;
+    }
+    if (!(out->dtype == MME_HIP_FP32 || out->dtype == MME_HIP_BF16 || is_fp8(out->dtype))) return fail(h, MME_HIP_EINVAL, "Unsupported type");
+    if (epi->rounding_mode == MME_HIP_RM_STOCHASTIC || epi->rounding_mode == MME_HIP_RM_STOCHASTIC_AND_NEAREST)
+        return fail(h, MME_HIP_EUNSUPPORTED, "stochastic rounding is not built for the fused epilogue");
+    if (epi->scale_exp < -126 || epi->scale_exp > 126) return fail(h, MME_HIP_EINVAL, "scale exponent out of range");
+    return MME_HIP_OK;
+}
+
+CastParams make_cast(int dtype, unsigned bias, int mode, int rm, int clip, int clip_inf, int ftz, int relu, int scale_exp)
+{
+    CastParams c;
+    c.dtype = dtype == MME_HIP_FP32_IEEE ? DT_FP32 : dtype;
+    c.exp_bias = (int) bias;
+    c.inf_nan_mode = mode;
+    c.rm = rm;
+    c.clip_fp = clip;
+    c.clip_inf_in = clip_inf;
+    c.ftz = ftz;
+    c.relu = relu;
+    c.has_scale = scale_exp != 0;
+    uint32_t bits = (uint32_t) (scale_exp + 127) << 23;
+    memcpy(&c.scale, &bits, 4);
+    return c;
+}
+
+float pow2f(int e)
+{
+    uint32_t bits = (uint32_t) (e + 127) << 23;
+    float    f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+// ---- fp8 operands: fold Gaudi's exponent bias into a power of two, decide whether the hardware formats suffice -------
+struct Fp8Plan
+{
+    int fold_exp = 0;     // accumulators are multiplied by 2^fold_exp
+    int scan_kind[2] = {-1, -1}; // -1: every code is exact in the hardware format; 0 / 1: mask kind to scan for
+};
+
+Fp8Plan plan_fp8(const mme_hip_tensor* a, const mme_hip_tensor* b)
+{
+    Fp8Plan               p;
+    const mme_hip_tensor* t[2] = {a, b};
+    for (int i = 0; i < 2; i++)
+    {
+        if (t[i]->dtype == MME_HIP_FP8_143)
+        {
+            p.fold_exp += 7 - (int) t[i]->fp_bias; // hardware e4m3 has bias 7
+            // full mode: exponent 15 is inf / NaN (finite 256..448 for the hardware); no-inf-nan mode: 0x7F is finite
+            // (NaN for the hardware); minimal mode is the hardware's own format
+            p.scan_kind[i] = t[i]->inf_nan_mode == 0 ? 0 : (t[i]->inf_nan_mode == 1 ? 1 : -1);
+        }
+        else
+        {
+            p.fold_exp += 15 - (int) t[i]->fp_bias; // hardware e5m2 has bias 15
+            // full mode is the hardware's own format; the other modes give finite meaning to exponent-31 codes
+            p.scan_kind[i] = t[i]->inf_nan_mode == 0 ? -1 : 0;
+        }
+    }
+    return p;
+}
+
+void set_plain_view(OperandView& v, const void* base, long long stride_f, long long stride_k, bool k_contig, int es, int extent_contig,
+                    const long long bstride[3])
+{
+    memset(&v, 0, sizeof v);
+    v.base = (const char*) base;
+    v.kind = VIEW_PLAIN;
+    v.stride_f = stride_f;
+    v.stride_k = stride_k;
+    v.k_contig = k_contig;
+    const int       kv = 16 / es;
+    const long long other = k_contig ? stride_f : stride_k;
+    bool            ok = ((uintptr_t) base % 16 == 0) && (other % kv == 0) && (extent_contig % kv == 0);
+    for (int i = 0; i < 3; i++)
+    {
+        v.batch_stride[i] = bstride[i];
+        ok = ok && (bstride[i] % kv == 0);
+    }
+    v.vec_ok = ok;
+}
+
+int ensure_flag(mme_hip_handle h)
+{
+    if (!h->flag.p) HIP_TRY(h, h->flag.reserve(256));
+    return MME_HIP_OK;
+}
+
+// Runs one contraction, taking care of fp8 operands: native MFMA formats when every code is exact there, otherwise an
+// exact fp8 -> bf16 decode followed by the bf16 kernel.  Both variants are enqueued, a device flag picks one, so the
+// call never waits for the device.
+int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, const mme_hip_tensor* tb, const void* a_base,
+                    const void* b_base)
+{
+    g.skip_flag = nullptr;
+    g.skip_if = 0;
+    g.split_k = gemm_pick_split_k(g, h->num_cus);
+    g.workspace = nullptr;
+    if (g.split_k > 1)
+    {
+        HIP_TRY(h, h->split_ws.reserve(gemm_workspace_bytes(g)));
+        g.workspace = (float*) h->split_ws.p;
+    }
+    if (!is_fp8(g.dtype))
+    {
+        HIP_TRY(h, launch_gemm(g, h->stream));
+        return MME_HIP_OK;
+    }
+    const Fp8Plan plan = plan_fp8(ta, tb);
+    g.fmt_a = ta->dtype == MME_HIP_FP8_152;
+    g.fmt_b = tb->dtype == MME_HIP_FP8_152;
+    const int fold = plan.fold_exp;
+    // alpha so far holds the caller's descale (or 1); fold the bias difference into the same multiplication
+    {
+        uint32_t bits;
+        memcpy(&bits, &g.epi.alpha, 4);
+        int e = g.epi.has_alpha ? (int) ((bits >> 23) & 0xFF) - 127 : 0;
+        e += fold;
+        if (e < -126 || e > 126) return fail(h, MME_HIP_EINVAL, "exponent bias and scale exponents exceed the fp32 range");
+        g.epi.alpha = pow2f(e);
+        g.epi.has_alpha = e != 0;
+    }
+    const bool need_scan = (plan.scan_kind[0] >= 0 || plan.scan_kind[1] >= 0) && h->fp8_specials_policy == 0;
+    if (!need_scan)
+    {
+        HIP_TRY(h, launch_gemm(g, h->stream));
+        return MME_HIP_OK;
+    }
+    // scan -> flag; native kernel runs when flag == 0; decode + bf16 kernel run when flag != 0
+    if (int rc = ensure_flag(h)) return rc;
+    uint32_t* flag = (uint32_t*) h->flag.p;
+    HIP_TRY(h, launch_fill_u32(flag, 0u, 1, h->stream));
+    const mme_hip_tensor* t[2] = {ta, tb};
+    const void*           base[2] = {a_base, b_base};
+    for (int i = 0; i < 2; i++)
+        if (plan.scan_kind[i] >= 0)
+            HIP_TRY(h, launch_fp8_special_scan(flag, base[i], span_elements(t[i]), t[i]->dtype == MME_HIP_FP8_143 ? 3 : 2,
+                                               plan.scan_kind[i], h->stream));
+    g.skip_flag = flag;
+    g.skip_if = 1; // native variant: skipped when the flag is set
+    HIP_TRY(h, launch_gemm(g, h->stream));
+
+    const size_t na = span_elements(ta), nb = span_elements(tb);
+    const size_t na_pad = (na + 7) & ~(size_t) 7;
+    HIP_TRY(h, h->decode_ws.reserve((na_pad + nb + 8) * 2));
+    uint16_t* da = (uint16_t*) h->decode_ws.p;
+    uint16_t* db = da + na_pad;
+    HIP_TRY(h, launch_fp8_to_bf16(da, (const uint8_t*) a_base, na, ta->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) ta->fp_bias,
+                                  ta->inf_nan_mode, flag, h->stream));
+    HIP_TRY(h, launch_fp8_to_bf16(db, (const uint8_t*) b_base, nb, tb->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) tb->fp_bias,
+                                  tb->inf_nan_mode, flag, h->stream));
+    GemmProblem g2 = g;
+    g2.dtype = DT_BF16;
+    g2.A.base = (const char*) da;
+    g2.B.base = (const char*) db;
+    // the decoded copies keep the operands' layout; vector legality: 8 bf16 per 16 bytes is a weaker requirement than
+    // 16 fp8 per 16 bytes on every stride, and both copies start 16-byte aligned
+    {
+        uint32_t bits;
+        memcpy(&bits, &g.epi.alpha, 4);
+        int e = g.epi.has_alpha ? (int) ((bits >> 23) & 0xFF) - 127 : 0;
+        e -= fold; // decoded operands carry their true values
+        g2.epi.alpha = pow2f(e);
+        g2.epi.has_alpha = e != 0;
+    }
+    g2.skip_if = 0; // decoded variant: skipped when the flag is clear
+    g2.split_k = g.split_k;
+    HIP_TRY(h, launch_gemm(g2, h->stream));
+    return MME_HIP_OK;
+}
+
+int fill_epilogue(mme_hip_handle h, GemmEpilogue& e, const mme_hip_tensor* out, const mme_hip_epilogue* epi)
+{
+    memset(&e, 0, sizeof e);
+    e.out = out->data;
+    e.out_dtype = out->dtype == MME_HIP_FP32_IEEE ? DT_FP32 : out->dtype;
+    e.alpha = 1.0f;
+    if (epi)
+    {
+        e.fused = 1;
+        e.cast = make_cast(out->dtype, out->fp_bias, out->inf_nan_mode, epi->rounding_mode, epi->clip_fp, epi->clip_inf_in,
+                           epi->flush_denorms, epi->relu, 0);
+        e.fast_cast = cast_params_fast(e.cast);
+        e.alpha = pow2f(epi->scale_exp);
+        e.has_alpha = epi->scale_exp != 0;
+        e.col_exp = epi->col_scale_exp;
+    }
+    (void) h;
+    return MME_HIP_OK;
+}
+} // namespace
+
+// =====================================================================================================================
+extern "C" {
+
+const char* mme_hip_version(void) { return "mme-hip 0.1 gfx950"; }
+
+const char* mme_hip_last_error(mme_hip_handle h) { return h ? h->error.c_str() : g_create_error.c_str(); }
+
+int mme_hip_create(mme_hip_handle* out, int chip, int max_tensor_dims, int max_conv_dims, unsigned seed, uint32_t lfsr_num_regs,
+                   const uint32_t* lfsr, uint32_t polynomial)
+{
+    if (!out) return fail(nullptr, MME_HIP_EINVAL, "got null pointer");
+    *out = nullptr;
+    if (max_tensor_dims != MME_HIP_MAX_TENSOR_DIMS || max_conv_dims != MME_HIP_MAX_CONV_DIMS)
+        return fail(nullptr, MME_HIP_EINVAL, "dynamic value different than static value");
+    if (chip != MME_HIP_CHIP_GAUDI3)
+    {
+        if (chip == MME_HIP_CHIP_GAUDI || chip == MME_HIP_CHIP_GAUDI2)
+            return fail(nullptr, MME_HIP_EUNSUPPORTED, "only the Gaudi3 numerics are built in this library");
+        return fail(nullptr, MME_HIP_EINVAL, "unknown chip type");
+    }
+    mme_hip_calc* h = new (std::nothrow) mme_hip_calc;
+    if (!h) return fail(nullptr, MME_HIP_ENOMEM, "out of host memory");
+    hipError_t e = hipGetDevice(&h->device);
+    if (e == hipSuccess)
+    {
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, h->device);
+        if (e == hipSuccess)
+        {
+            h->num_cus = prop.multiProcessorCount;
+            if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            {
+                std::string arch = prop.gcnArchName;
+                delete h;
+                return fail(nullptr, MME_HIP_EHIP, "this library holds gfx950 code objects only, device is %s", arch.c_str());
+            }
+        }
+    }
+    if (e == hipSuccess) e = hipStreamCreateWithFlags(&h->own_stream, hipStreamNonBlocking);
+    if (e != hipSuccess)
+    {
+        delete h;
+        return fail(nullptr, MME_HIP_EHIP, "no usable HIP device: %s", hipGetErrorString(e));
+    }
+    h->stream = h->own_stream;
+    // LFSR registers and polynomial exactly as the reference seeds them (mme_reference_impl.cpp:146-170)
+    h->lfsr.resize(lfsr_num_regs);
+    for (uint32_t i = 0; i < lfsr_num_regs; i++) h->lfsr[i] = lfsr ? lfsr[i] : i + 2;
+    if (polynomial == 0)
+    {
+        std::mt19937                    gen(seed);
+        std::uniform_int_distribution<> distr(25, 63);
+        h->polynomial = (uint32_t) distr(gen);
+    }
+    else
+        h->polynomial = polynomial;
+    *out = h;
+    return MME_HIP_OK;
+}
+
+void mme_hip_destroy(mme_hip_handle h)
+{
+    if (!h) return;
+    if (h->own_stream)
+    {
+        (void) hipStreamSynchronize(h->own_stream);
+        (void) hipStreamDestroy(h->own_stream);
+    }
+    delete h;
+}
+
+int mme_hip_limit_num_of_threads(mme_hip_handle h, unsigned n)
+{
+    if (!h) return MME_HIP_EINVAL;
+    h->num_threads = n;
+    return MME_HIP_OK;
+}
+
+void* mme_hip_stream(mme_hip_handle h) { return h ? (void*) h->stream : nullptr; }
+
+int mme_hip_set_stream(mme_hip_handle h, void* s)
+{
+    if (!h) return MME_HIP_EINVAL;
+    h->stream = s ? (hipStream_t) s : h->own_stream;
+    return MME_HIP_OK;
+}
+
+int mme_hip_synchronize(mme_hip_handle h)
+{
+    if (!h) return MME_HIP_EINVAL;
+    HIP_TRY(h, hipStreamSynchronize(h->stream));
+    return MME_HIP_OK;
+}
+
+int mme_hip_set_fp8_specials_policy(mme_hip_handle h, int policy)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (policy != MME_HIP_FP8_SPECIALS_CHECK && policy != MME_HIP_FP8_SPECIALS_ASSUME_NONE)
+        return fail(h, MME_HIP_EINVAL, "unknown fp8 specials policy %d", policy);
+    h->fp8_specials_policy = policy;
+    return MME_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// batched GEMM
+// ---------------------------------------------------------------------------------------------------------------------
+int mme_hip_batch_gemm_dev(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, int op,
+                           const mme_hip_epilogue* epi)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (int rc = check_tensor(h, out, "output")) return rc;
+    if (int rc = check_tensor(h, x, "x")) return rc;
+    if (int rc = check_tensor(h, w, "w")) return rc;
+    if (op < MME_HIP_OP_AB || op > MME_HIP_OP_ATBT) return fail(h, MME_HIP_EINVAL, "invalid bgemm op %d", op);
+    if (int rc = check_operand_types(h, x, w)) return rc;
+    if (int rc = check_out_type(h, out, epi)) return rc;
+    for (int d = 2; d < 5; d++)
+        if (!((x->sizes[d] == out->sizes[d] || x->sizes[d] == 1) && (w->sizes[d] == out->sizes[d] || w->sizes[d] == 1)))
+            return fail(h, MME_HIP_EINVAL, "batch dims doesnt match !");
+    const int out_es = elem_size(out->dtype);
+    if (n_elements(x) == 0 || n_elements(w) == 0)
+    {
+        // zero common dimension: the output is all zeros (handleZeroCdCase, mme_reference_impl.cpp:204-216)
+        if (n_elements(x) != n_elements(w)) return fail(h, MME_HIP_EINVAL, "One of the input tensors is zero-size, while the other is not");
+        const size_t bytes = span_elements(out) * out_es;
+        if (bytes % 4) return fail(h, MME_HIP_EUNSUPPORTED, "zero-size contraction into an output whose byte size is not a multiple of 4");
+        HIP_TRY(h, launch_fill_u32((uint32_t*) out->data, 0u, bytes / 4, h->stream));
+        return MME_HIP_OK;
+    }
+    const bool ta = (op == MME_HIP_OP_ATB || op == MME_HIP_OP_ATBT);
+    const bool tb = (op == MME_HIP_OP_ABT || op == MME_HIP_OP_ATBT);
+    const int  M = ta ? x->sizes[0] : x->sizes[1];
+    const int  Ka = ta ? x->sizes[1] : x->sizes[0];
+    const int  Kb = tb ? w->sizes[0] : w->sizes[1];
+    const int  N = tb ? w->sizes[1] : w->sizes[0];
+    if (Ka != Kb) return fail(h, MME_HIP_EINVAL, "Common dim doesnt match between input A\\B");
+    if ((int) out->sizes[0] != N) return fail(h, MME_HIP_EINVAL, "output width doesnt match to inputB width");
+    if ((int) out->sizes[1] != M) return fail(h, MME_HIP_EINVAL, "output height doesnt match to inputA height");
+
+    GemmProblem g;
+    memset(&g, 0, sizeof g);
+    g.dtype = x->dtype;
+    g.M = M;
+    g.N = N;
+    g.K = Ka;
+    const int es = elem_size(x->dtype);
+    long long abs_[3], bbs[3];
+    for (int d = 0; d < 3; d++)
+    {
+        g.batch[d] = out->sizes[d + 2];
+        abs_[d] = x->sizes[d + 2] == 1 ? 0 : x->strides[d + 2];
+        bbs[d] = w->sizes[d + 2] == 1 ? 0 : w->strides[d + 2];
+    }
+    // A(m, k): x[m * s1 + k] or, transposed, x[k * s1 + m];   B(n, k): w[k * s1 + n] or, transposed, w[n * s1 + k]
+    set_plain_view(g.A, x->data, ta ? 1 : x->strides[1], ta ? x->strides[1] : 1, !ta, es, ta ? M : Ka, abs_);
+    set_plain_view(g.B, w->data, tb ? w->strides[1] : 1, tb ? 1 : w->strides[1], tb, es, tb ? Kb : N, bbs);
+    if (int rc = fill_epilogue(h, g.epi, out, epi)) return rc;
+    g.epi.ld = out->strides[1];
+    for (int d = 0; d < 3; d++) g.epi.batch_stride[d] = out->strides[d + 2];
+    return run_contraction(h, g, x, w, x->data, w->data);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// convolution
+// ---------------------------------------------------------------------------------------------------------------------
+int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w,
+                            const mme_hip_tensor* y, const mme_hip_conv_params* cp, int op, const mme_hip_epilogue* epi)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (!cp) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    if (op == MME_HIP_OP_TRANSPOSED_DEDX || op == MME_HIP_OP_DETERMINISTIC_DEDW)
+        return fail(h, MME_HIP_EUNSUPPORTED, "op %d is not built in this library", op);
+    if (op != MME_HIP_OP_FWD && op != MME_HIP_OP_DEDX && op != MME_HIP_OP_DEDW) return fail(h, MME_HIP_EINVAL, "invalid operation");
+    // operand roles (mme_reference_impl.cpp:611-655): fwd A=x B=w; dedx A=y B=w; dedw A=x B=y
+    const mme_hip_tensor* A = op == MME_HIP_OP_DEDX ? y : x;
+    const mme_hip_tensor* B = op == MME_HIP_OP_DEDW ? y : w;
+    if (int rc = check_tensor(h, out, "output")) return rc;
+    if (int rc = check_tensor(h, A, "inputA")) return rc;
+    if (int rc = check_tensor(h, B, "inputB")) return rc;
+    if (int rc = check_operand_types(h, A, B)) return rc;
+    if (int rc = check_out_type(h, out, epi)) return rc;
+    for (int i = 0; i < 4; i++)
+        if (cp->conv_stride[i] < 1 || cp->dilation[i] < 1) return fail(h, MME_HIP_EINVAL, "convolution stride and dilation must be positive");
+
+    const mme_hip_tensor* wt = op == MME_HIP_OP_DEDW ? out : w; // weight-shaped  [K, C, S, R, Q]
+    const mme_hip_tensor* yt = op == MME_HIP_OP_FWD ? out : y;  // output-shaped  [K, W', H', D', B]
+    const mme_hip_tensor* xt = op == MME_HIP_OP_DEDX ? out : x; // input-shaped   [C, W, H, D, B]
+    const int Kc = wt->sizes[0], C = wt->sizes[1];
+    const int taps = wt->sizes[2] * wt->sizes[3] * wt->sizes[4];
+    if ((int) xt->sizes[0] != C) return fail(h, MME_HIP_EINVAL, "channel dims of x and w differ");
+    if ((int) yt->sizes[0] != Kc) return fail(h, MME_HIP_EINVAL, "channel dims of y and w differ");
+    const long long y_pix = (long long) yt->sizes[1] * yt->sizes[2] * yt->sizes[3] * yt->sizes[4];
+    const long long x_pix = (long long) xt->sizes[1] * xt->sizes[2] * xt->sizes[3] * xt->sizes[4];
+    if (y_pix >= (1ll << 31) || x_pix >= (1ll << 31) || (long long) taps * std::max(C, Kc) >= (1ll << 31))
+        return fail(h, MME_HIP_EINVAL, "convolution extents exceed 2^31");
+    if (n_elements(out) == 0) return MME_HIP_OK;
+
+    // dense weight tensor and row-collapsible outputs keep the addressing linear
+    {
+        uint64_t acc = 1;
+        for (int d = 0; d < 5; d++)
+        {
+            if (wt->sizes[d] > 1 && wt->strides[d] != acc) return fail(h, MME_HIP_EUNSUPPORTED, "strided weight tensors are not built in this library");
+            acc *= wt->sizes[d];
+        }
+    }
+    if (!rows_collapsible(out)) return fail(h, MME_HIP_EUNSUPPORTED, "output tensors with non-collapsible row strides are not built");
+    if (op == MME_HIP_OP_DEDW && !rows_collapsible(y)) return fail(h, MME_HIP_EUNSUPPORTED, "dedw needs a row-collapsible dy tensor");
+
+    const int es = elem_size(A->dtype);
+    const int kv = 16 / es;
+
+    GemmProblem g;
+    memset(&g, 0, sizeof g);
+    g.dtype = A->dtype;
+    g.batch[0] = g.batch[1] = g.batch[2] = 1;
+    const long long zero3[3] = {0, 0, 0};
+
+    auto conv_view = [&](OperandView& v, const mme_hip_tensor* src, const mme_hip_tensor* pixels, int nch, int pix_is_f, int gather_y) {
+        memset(&v, 0, sizeof v);
+        v.base = (const char*) src->data;
+        v.kind = VIEW_CONV;
+        v.pix_is_f = pix_is_f;
+        v.gather_y = gather_y;
+        v.nch = nch;
+        v.k_contig = pix_is_f; // channels are contiguous; they run along k when pixels run along f
+        bool ok = ((uintptr_t) src->data % 16 == 0) && (nch % kv == 0);
+        for (int d = 0; d < 4; d++)
+        {
+            v.grid[d] = pixels->sizes[d + 1];
+            v.src[d] = src->sizes[d + 1];
+            v.src_stride[d] = src->strides[d + 1];
+            v.cstride[d] = cp->conv_stride[d];
+            v.dil[d] = cp->dilation[d];
+            v.pad[d] = cp->padding[d];
+            ok = ok && (src->strides[d + 1] % kv == 0);
+        }
+        for (int d = 0; d < 3; d++) v.ktap[d] = wt->sizes[d + 2];
+        v.vec_ok = ok;
+    };
+
+    if (op == MME_HIP_OP_FWD)
+    {
+        // Y[pix][k] = sum_{tap, c} X[pos(pix, tap)][c] * W[(tap * C + c)][k]
+        g.M = (int) y_pix;
+        g.N = Kc;
+        g.K = taps * C;
+        conv_view(g.A, x, out, C, 1, 0);
+        set_plain_view(g.B, w->data, 1, Kc, false, es, Kc, zero3);
+    }
+    else if (op == MME_HIP_OP_DEDX)
+    {
+        // dX[pix][c] = sum_{tap, k} dY[src(pix, tap)][k] * W[(tap * C + c)][k]     (gather form of col2im)
+        g.M = (int) x_pix;
+        g.N = C;
+        g.K = taps * Kc;
+        conv_view(g.A, y, out, Kc, 1, 1);
+        memset(&g.B, 0, sizeof g.B);
+        g.B.base = (const char*) w->data;
+        g.B.kind = VIEW_TAPPED;
+        g.B.k_contig = 1;
+        g.B.stride_f = Kc;
+        g.B.stride_k = 1;
+        g.B.tap_stride = (long long) Kc * C;
+        g.B.nch = Kc;
+        g.B.vec_ok = ((uintptr_t) w->data % 16 == 0) && (Kc % kv == 0);
+    }
+    else
+    {
+        // dW[(tap * C + c)][k] = sum_pix X[pos(pix, tap)][c] * dY[pix][k]
+        g.M = taps * C;
+        g.N = Kc;
+        g.K = (int) y_pix;
+        conv_view(g.A, x, y, C, 0, 0);
+        set_plain_view(g.B, y->data, 1, y->strides[1], false, es, Kc, zero3);
+    }
+    if (int rc = fill_epilogue(h, g.epi, out, epi)) return rc;
+    g.epi.ld = out->strides[1];
+    return run_contraction(h, g, A, B, A->data, B->data);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// activation / casts
+// ---------------------------------------------------------------------------------------------------------------------
+int mme_hip_activation_dev(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* acc, int relu, int rm, int clip_fp,
+                           int clip_inf_in, int flush_denorms, int stochastic_ftz)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (int rc = check_tensor(h, out, "output")) return rc;
+    if (int rc = check_tensor(h, acc, "acc")) return rc;
+    if (acc->dtype != MME_HIP_FP32) return fail(h, MME_HIP_EINVAL, "acc element type should be fp32");
+    if (acc->dim != out->dim) return fail(h, MME_HIP_EINVAL, "dims number of outputTensor doesnt match acc output");
+    for (int d = 0; d < 5; d++)
+        if (acc->sizes[d] != out->sizes[d]) return fail(h, MME_HIP_EINVAL, "sizes of output Tensot doesnt match acc output");
+    if (!(out->dtype == MME_HIP_FP32 || out->dtype == MME_HIP_BF16 || is_fp8(out->dtype))) return fail(h, MME_HIP_EINVAL, "Unsupported type");
+    if (rm == MME_HIP_RM_STOCHASTIC || rm == MME_HIP_RM_STOCHASTIC_AND_NEAREST || stochastic_ftz)
+        return fail(h, MME_HIP_EUNSUPPORTED, "stochastic rounding / stochastic flush are not built in this library");
+    if (!(rm == 0 || rm == 1 || rm == 2 || rm == 3 || rm == 6)) return fail(h, MME_HIP_EINVAL, "invalid rounding mode %d", rm);
+    // the reference converts the first getSizeInElements() elements of both flat buffers (:1155)
+    const size_t n = n_elements(acc);
+    if (relu) HIP_TRY(h, launch_relu_inplace((float*) acc->data, n, h->stream));
+    const CastParams c = make_cast(out->dtype, out->fp_bias, out->inf_nan_mode, rm, clip_fp, clip_inf_in, flush_denorms, 0, 0);
+    HIP_TRY(h, launch_cast_from_fp32(out->data, (const float*) acc->data, n, c, nullptr, 0, h->stream));
+    return MME_HIP_OK;
+}
+
+int mme_hip_cast_from_fp32_dev(mme_hip_handle h, void* out, int out_dtype, unsigned out_fp_bias, int out_inf_nan_mode, const float* in,
+                               size_t n, int scale_exp, const int32_t* col_scale_exp, size_t n_cols, int relu, int rm, int clip_fp,
+                               int clip_inf_in, int flush_denorms)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (!(out_dtype == MME_HIP_FP32 || out_dtype == MME_HIP_BF16 || is_fp8(out_dtype))) return fail(h, MME_HIP_EINVAL, "Unsupported type");
+    if (!(rm == 0 || rm == 1 || rm == 2 || rm == 3 || rm == 6))
+        return fail(h, rm == 4 || rm == 7 ? MME_HIP_EUNSUPPORTED : MME_HIP_EINVAL, "rounding mode %d is not available here", rm);
+    if (scale_exp < -126 || scale_exp > 126) return fail(h, MME_HIP_EINVAL, "scale exponent out of range");
+    if (col_scale_exp && n_cols == 0) return fail(h, MME_HIP_EINVAL, "n_cols must be positive with per-column scales");
+    if (n && (!out || !in)) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    const CastParams c = make_cast(out_dtype, out_fp_bias, out_inf_nan_mode, rm, clip_fp, clip_inf_in, flush_denorms, relu, scale_exp);
+    HIP_TRY(h, launch_cast_from_fp32(out, in, n, c, col_scale_exp, n_cols, h->stream));
+    return MME_HIP_OK;
+}
+
+int mme_hip_cast_to_fp32_dev(mme_hip_handle h, float* out, const void* in, int in_dtype, unsigned in_fp_bias, int in_inf_nan_mode, size_t n,
+                             int scale_exp, const int32_t* col_scale_exp, size_t n_cols)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (!(in_dtype == MME_HIP_BF16 || is_fp8(in_dtype))) return fail(h, MME_HIP_EINVAL, "Unsupported type");
+    if (scale_exp < -126 || scale_exp > 126) return fail(h, MME_HIP_EINVAL, "scale exponent out of range");
+    if (col_scale_exp && n_cols == 0) return fail(h, MME_HIP_EINVAL, "n_cols must be positive with per-column scales");
+    if (n && (!out || !in)) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    HIP_TRY(h, launch_cast_to_fp32(out, in, in_dtype, (int) in_fp_bias, in_inf_nan_mode, n, pow2f(scale_exp), scale_exp != 0, col_scale_exp,
+                                   n_cols, h->stream));
+    return MME_HIP_OK;
+}
+
+int mme_hip_absmax_dev(mme_hip_handle h, float* out_absmax, const float* in, size_t n)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (!out_absmax || (n && !in)) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    HIP_TRY(h, launch_absmax(out_absmax, in, n, h->stream));
+    return MME_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// host-pointer entry points: stage through device memory, run the _dev form, copy back, synchronise
+// ---------------------------------------------------------------------------------------------------------------------
+namespace
+{
+struct Staged
+{
+    mme_hip_tensor t;
+    DeviceBuffer   buf;
+    void*          host = nullptr;
+    size_t         bytes = 0;
+};
+
+int stage_in(mme_hip_handle h, Staged& s, const mme_hip_tensor* src, bool copy)
+{
+    s.t = *src;
+    s.host = src->data;
+    s.bytes = (size_t) span_elements(src) * elem_size(src->dtype);
+    HIP_TRY(h, s.buf.reserve(s.bytes ? s.bytes : 16));
+    s.t.data = s.buf.p;
+    if (copy && s.bytes) HIP_TRY(h, hipMemcpyAsync(s.buf.p, s.host, s.bytes, hipMemcpyHostToDevice, h->stream));
+    return MME_HIP_OK;
+}
+int stage_out(mme_hip_handle h, Staged& s)
+{
+    if (s.bytes) HIP_TRY(h, hipMemcpyAsync(s.host, s.buf.p, s.bytes, hipMemcpyDeviceToHost, h->stream));
+    return MME_HIP_OK;
+}
+bool has_gaps(const mme_hip_tensor* t) { return span_elements(t) != n_elements(t); }
+} // namespace
+
+int mme_hip_batch_gemm(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, int op, int rm, int clip_fp,
+                       int clip_fp_inf_in)
+{
+    (void) rm; // the Gaudi3 tree hard-codes round-to-zero; clipFp is dropped by its FMA classes (gaudi3_fma.h:43,79)
+    (void) clip_fp;
+    (void) clip_fp_inf_in;
+    if (!h) return MME_HIP_EINVAL;
+    if (int rc = check_tensor(h, out, "output")) return rc;
+    if (int rc = check_tensor(h, x, "x")) return rc;
+    if (int rc = check_tensor(h, w, "w")) return rc;
+    Staged so, sx, sw;
+    // a strided output keeps the bytes between its rows: copy them in first
+    if (int rc = stage_in(h, so, out, has_gaps(out))) return rc;
+    if (int rc = stage_in(h, sx, x, true)) return rc;
+    if (int rc = stage_in(h, sw, w, true)) return rc;
+    if (int rc = mme_hip_batch_gemm_dev(h, &so.t, &sx.t, &sw.t, op, nullptr)) return rc;
+    if (int rc = stage_out(h, so)) return rc;
+    HIP_TRY(h, hipStreamSynchronize(h->stream));
+    return MME_HIP_OK;
+}
+
+int mme_hip_convolution(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, const mme_hip_tensor* y,
+                        const mme_hip_conv_params* cp, int op, int rm, int clip_fp, int clip_fp_inf_in)
+{
+    (void) rm; // reaches only col2im's additions in the reference; all taps share one accumulator here
+    (void) clip_fp;
+    (void) clip_fp_inf_in;
+    if (!h) return MME_HIP_EINVAL;
+    if (op != MME_HIP_OP_FWD && op != MME_HIP_OP_DEDX && op != MME_HIP_OP_DEDW)
+        return mme_hip_convolution_dev(h, out, x, w, y, cp, op, nullptr); // reports the error
+    const mme_hip_tensor* A = op == MME_HIP_OP_DEDX ? y : x;
+    const mme_hip_tensor* B = op == MME_HIP_OP_DEDW ? y : w;
+    if (int rc = check_tensor(h, out, "output")) return rc;
+    if (int rc = check_tensor(h, A, "inputA")) return rc;
+    if (int rc = check_tensor(h, B, "inputB")) return rc;
+    Staged so, sa, sb;
+    if (int rc = stage_in(h, so, out, has_gaps(out))) return rc;
+    if (int rc = stage_in(h, sa, A, true)) return rc;
+    if (int rc = stage_in(h, sb, B, true)) return rc;
+    const mme_hip_tensor* dx = op == MME_HIP_OP_DEDX ? &so.t : &sa.t;
+    const mme_hip_tensor* dw = op == MME_HIP_OP_DEDW ? &so.t : &sb.t;
+    const mme_hip_tensor* dy = op == MME_HIP_OP_FWD ? &so.t : (op == MME_HIP_OP_DEDX ? &sa.t : &sb.t);
+    if (int rc = mme_hip_convolution_dev(h, &so.t, dx, dw, dy, cp, op, nullptr)) return rc;
+    if (int rc = stage_out(h, so)) return rc;
+    HIP_TRY(h, hipStreamSynchronize(h->stream));
+    return MME_HIP_OK;
+}
+
+int mme_hip_activation(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* acc, int relu, int rm, int clip_fp, int clip_inf_in,
+                       int flush_denorms, int stochastic_ftz)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (int rc = check_tensor(h, out, "output")) return rc;
+    if (int rc = check_tensor(h, acc, "acc")) return rc;
+    Staged so, sa;
+    if (int rc = stage_in(h, so, out, true)) return rc;
+    if (int rc = stage_in(h, sa, acc, true)) return rc;
+    if (int rc = mme_hip_activation_dev(h, &so.t, &sa.t, relu, rm, clip_fp, clip_inf_in, flush_denorms, stochastic_ftz)) return rc;
+    if (int rc = stage_out(h, so)) return rc;
+    if (relu)
+        if (int rc = stage_out(h, sa)) return rc; // relu rewrites acc in place in the reference (:683-686)
+    HIP_TRY(h, hipStreamSynchronize(h->stream));
+    return MME_HIP_OK;
+}
+
+int mme_hip_memory_write(mme_hip_handle h, const mme_hip_tensor* memory, const mme_hip_tensor* mme_out, int reduction_op, int reduction_rm,
+                         int clip_fp)
+{
+    (void) reduction_rm;
+    (void) clip_fp;
+    if (!h) return MME_HIP_EINVAL;
+    if (!memory || !mme_out) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    if (reduction_op != MME_HIP_REDUCTION_NONE) return fail(h, MME_HIP_EUNSUPPORTED, "memory-write reductions are not built in this library");
+    // reduction none: a byte copy of the destination tensor's size (mme_reference_impl.cpp:725-729)
+    const size_t bytes = (size_t) span_elements(memory) * elem_size(memory->dtype);
+    if (bytes) memmove(memory->data, mme_out->data, bytes);
+    return MME_HIP_OK;
+}
+
+} // extern "C"

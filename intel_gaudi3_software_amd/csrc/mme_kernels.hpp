@@ -1,0 +1,99 @@
+// mme_kernels.hpp -- internal (C++) interface between the C ABI layer and the HIP kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+#include "mme_numeric.hpp"
+
+namespace mme
+{
+// ---- elementwise (cast_kernels.hip) ---------------------------------------------------------------------------
+hipError_t launch_cast_from_fp32(void* out, const float* in, size_t n, const CastParams& p, const int32_t* col_exp,
+                                 size_t n_cols, hipStream_t s);
+hipError_t launch_cast_to_fp32(float* out, const void* in, int dtype, int bias, int mode, size_t n, float scale,
+                               int has_scale, const int32_t* col_exp, size_t n_cols, hipStream_t s);
+hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s);
+hipError_t launch_absmax(float* out, const float* in, size_t n, hipStream_t s);
+
+// ---- contraction (gemm_kernels.hip) ---------------------------------------------------------------------------
+//
+// Every contraction of the path is C[f_a][f_b] = sum_k A(f_a, k) * B(f_b, k) over one "view" per operand.
+// A view maps (free index f, reduction index k) to an element address, either as a plain strided matrix or through
+// the im2col / col2im addressing of the reference (mme/mme_reference/im2col.cpp:134-172).
+
+enum : int
+{
+    VIEW_PLAIN = 0,  // base + f * stride_f + k * stride_k (+ batch offset)
+    VIEW_CONV = 1,   // (pixel, tap, channel) gather, see below
+    VIEW_TAPPED = 2  // k = tap * nch + ch:  base + f * stride_f + ch * stride_k + tap * tap_stride  (weights of dedx)
+};
+
+struct OperandView
+{
+    const char* base;
+    int         kind;
+    int         k_contig; // 1: consecutive k are adjacent in memory, 0: consecutive f are
+    int         vec_ok;   // 16-byte vector loads along the contiguous index are legal and never straddle a boundary
+    // VIEW_PLAIN
+    long long stride_f, stride_k; // elements
+    long long batch_stride[3];    // elements, 0 where the operand is broadcast
+    long long tap_stride;         // VIEW_TAPPED only
+    // VIEW_CONV: element = src[pos(pixel, tap)][channel]
+    int       pix_is_f;   // 1: f = pixel, k = tap * nch + channel;  0: k = pixel, f = tap * nch + channel
+    int       gather_y;   // 0: pos = pixel * stride + tap * dilation - padding (read x at an output pixel)
+                          // 1: pos = (pixel + padding - tap * dilation) / stride, exact division only (read dy at an
+                          //    input pixel: the gather form of col2im)
+    int       nch;        // channels per tap
+    int       grid[4];    // extents of the pixel index space (dims 1..4 of the tensor that enumerates pixels)
+    int       src[4];     // extents of dims 1..4 of the tensor being read
+    long long src_stride[4];
+    int       ktap[3];    // S, R, Q
+    int       cstride[4], dil[4], pad[4];
+};
+
+struct GemmEpilogue
+{
+    void*          out;
+    long long      ld;              // elements between consecutive f_a rows of the output
+    long long      batch_stride[3];
+    int            out_dtype;       // DT_*
+    CastParams     cast;            // used when fused != 0
+    int            fused;           // 0: raw fp32 accumulators (times alpha)
+    float          alpha;           // exact power of two folded into the accumulators (fp8 bias fold, descale)
+    int            has_alpha;
+    const int32_t* col_exp;         // per f_b power-of-two exponents or NULL
+    int            fast_cast;
+};
+
+struct GemmProblem
+{
+    int          dtype;      // operand element type (DT_*); fp8 operands may differ in flavour
+    int          fmt_a, fmt_b; // fp8 only: 0 = 4-bit exponent (e4m3), 1 = 5-bit exponent (e5m2)
+    int          M, N, K;    // extents of f_a, f_b, k
+    int          batch[3];
+    OperandView  A, B;
+    GemmEpilogue epi;
+    int          split_k;    // >1: partial sums go to workspace and are reduced in a fixed order
+    float*       workspace;  // split_k * batch * M * N floats
+    // device-side predicate: when skip_flag != NULL the whole launch returns at once if (*skip_flag != 0) == skip_if.
+    // Lets the fp8 path enqueue "native fp8" and "decoded bf16" variants back to back without a host round trip.
+    const uint32_t* skip_flag;
+    int             skip_if;
+};
+
+size_t     gemm_workspace_bytes(const GemmProblem& p);
+int        gemm_pick_split_k(const GemmProblem& p, int num_cus);
+hipError_t launch_gemm(const GemmProblem& p, hipStream_t s);
+
+// flags every exponent-all-ones code of an fp8 buffer (inf / NaN in Gaudi's full mode, finite for the hardware's
+// e4m3): *flag |= 1.  mask_kind 0: any code with all exponent bits set; 1: only 0x7F / 0xFF.
+hipError_t launch_fp8_special_scan(uint32_t* flag, const void* data, size_t n, int man_bits, int mask_kind, hipStream_t s);
+
+// dense or strided 5-d fp8 -> bf16 exact decode (used when the hardware's fp8 formats cannot represent the operand)
+// run_flag (device, may be NULL): the kernel does nothing when *run_flag == 0
+hipError_t launch_fp8_to_bf16(uint16_t* out, const uint8_t* in, size_t n, int man_bits, int bias, int mode, const uint32_t* run_flag,
+                              hipStream_t s);
+// one-lane fill of n 32-bit cells (kernels instead of memset nodes keep call sequences graph-capturable)
+hipError_t launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s);
+
+} // namespace mme

@@ -1,0 +1,93 @@
+"""Convolution fwd / dedx / dedw on the GPU against the oracle (reference im2col + GEMM + col2im restated)."""
+import numpy as np
+import pytest
+
+from intel_gaudi3_software_amd import ConvolutionParams, MmeSimTensor, abi
+from helpers import A, TOL, desc, random_operand, rel_frobenius
+
+pytestmark = pytest.mark.gpu
+
+
+def _osz(i, k, p, s, d):
+    return (i + 2 * p - d * (k - 1) - 1) // s + 1
+
+
+# (C, K, W, H, D, B, S, R, Q, padding, stride, dilation, dim)
+CASES = [
+    (3, 4, 5, 5, 1, 2, 3, 3, 1, (1, 1, 0), (2, 2, 1), (1, 1, 1), 2),    # odd channels: element-wise loads
+    (4, 3, 7, 6, 1, 2, 3, 2, 1, (2, 0, 0), (1, 2, 1), (2, 1, 1), 2),    # dilation, asymmetric padding
+    (2, 3, 5, 4, 3, 1, 2, 2, 2, (1, 0, 1), (1, 1, 1), (1, 2, 1), 3),    # 3-d
+    (16, 32, 9, 8, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),  # vector loads
+    (32, 16, 12, 10, 1, 2, 3, 3, 1, (1, 1, 0), (2, 2, 1), (1, 1, 1), 2),  # vector loads, stride 2 (dedx skips)
+    (16, 16, 6, 6, 1, 1, 1, 1, 1, (0, 0, 0), (1, 1, 1), (1, 1, 1), 2),  # 1x1
+]
+
+
+def _run(calc, orc, case, dt, bias, op, device):
+    import torch
+    (C, K, W, H, D, B, S, R, Q, pad, st, dil, dim) = case
+    rng = np.random.default_rng(100 + op)
+    Wo, Ho, Do = _osz(W, S, pad[0], st[0], dil[0]), _osz(H, R, pad[1], st[1], dil[1]), _osz(D, Q, pad[2], st[2], dil[2])
+    xs, ws, ys = [C, W, H, D, B], [K, C, S, R, Q], [K, Wo, Ho, Do, B]
+    x = random_operand(rng, dt, int(np.prod(xs)), orc, bias)
+    w = random_operand(rng, dt, int(np.prod(ws)), orc, bias, scale=0.3)
+    y = random_operand(rng, dt, int(np.prod(ys)), orc, bias, scale=0.5)
+    osz = {abi.OP_FWD: ys, abi.OP_DEDX: xs, abi.OP_DEDW: ws}[op]
+    n = int(np.prod(osz))
+    want = np.zeros(n, np.float32)
+    p = abi.make_conv_params(dim, pad, st, dil)
+    dx, dw, dy, do = desc(x, xs, dt, bias), desc(w, ws, dt, bias), desc(y, ys, dt, bias), desc(want, osz, abi.FP32)
+    assert orc.orc_convolution(A(do), A(dx), A(dw), A(dy), A(p), op, 0) == 0, orc.orc_last_error()
+    cp = ConvolutionParams(dim, list(pad) + [0], list(st) + [1], list(dil) + [1])
+    if device:
+        conv = (lambda a: torch.from_numpy(a.view(np.int16) if dt == abi.BF16 else a).cuda())
+        tx, tw, ty = conv(x), conv(w), conv(y)
+        to = torch.zeros(n, dtype=torch.float32, device="cuda")
+        tens = {"x": MmeSimTensor(xs, 5, dt, tx, bias), "w": MmeSimTensor(ws, 5, dt, tw, bias), "y": MmeSimTensor(ys, 5, dt, ty, bias)}
+        out = MmeSimTensor(osz, 5, abi.FP32, to)
+        calc.doConvolution(out, tens["x"], tens["w"], tens["y"], cp, op)
+        calc.synchronize()
+        got = to.cpu().numpy()
+    else:
+        got = np.zeros(n, np.float32)
+        calc.doConvolution(MmeSimTensor(osz, 5, abi.FP32, got), MmeSimTensor(xs, 5, dt, x, bias), MmeSimTensor(ws, 5, dt, w, bias),
+                           MmeSimTensor(ys, 5, dt, y, bias), cp, op)
+    return got, want
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP8_143, 7), (abi.FP32, 0)])
+@pytest.mark.parametrize("op", [abi.OP_FWD, abi.OP_DEDX, abi.OP_DEDW])
+def test_conv_vs_oracle(calc, orc, case, dt, bias, op):
+    got, want = _run(calc, orc, case, dt, bias, op, device=(case[0] % 16 == 0))
+    assert rel_frobenius(got, want) <= TOL[dt]
+    # positions the reference leaves at exactly zero (dedx with stride > 1) must be exactly zero here as well
+    assert np.all(got[want == 0] == 0) or op != abi.OP_DEDX
+
+
+def test_conv_adjoint_identities(calc, orc):
+    """<dY, fwd(X, W)> = <dedx(dY, W), X> = <dedw(X, dY), W> on a shape too large for the oracle to do quickly."""
+    import torch
+    rng = np.random.default_rng(77)
+    C, K, W, H, B = 64, 64, 28, 28, 8
+    xs, ws, ys = [C, W, H, 1, B], [K, C, 3, 3, 1], [K, W, H, 1, B]
+    from helpers import bf16_bits_to_f32, to_bf16_bits
+    x = to_bf16_bits(rng.standard_normal(int(np.prod(xs))))
+    w = to_bf16_bits(rng.standard_normal(int(np.prod(ws))) * 0.1)
+    dy = to_bf16_bits(rng.standard_normal(int(np.prod(ys))))
+    conv = lambda a: torch.from_numpy(a.view(np.int16)).cuda()
+    tx, tw, ty = conv(x), conv(w), conv(dy)
+    X, Wt, Y = MmeSimTensor(xs, 5, abi.BF16, tx), MmeSimTensor(ws, 5, abi.BF16, tw), MmeSimTensor(ys, 5, abi.BF16, ty)
+    cp = ConvolutionParams(2, [1, 1, 0, 0], [1, 1, 1, 1], [1, 1, 1, 1])
+    f = torch.zeros(int(np.prod(ys)), dtype=torch.float32, device="cuda")
+    gx = torch.zeros(int(np.prod(xs)), dtype=torch.float32, device="cuda")
+    gw = torch.zeros(int(np.prod(ws)), dtype=torch.float32, device="cuda")
+    calc.doConvolution(MmeSimTensor(ys, 5, abi.FP32, f), X, Wt, Y, cp, abi.OP_FWD)
+    calc.doConvolution(MmeSimTensor(xs, 5, abi.FP32, gx), X, Wt, Y, cp, abi.OP_DEDX)
+    calc.doConvolution(MmeSimTensor(ws, 5, abi.FP32, gw), X, Wt, Y, cp, abi.OP_DEDW)
+    calc.synchronize()
+    xf, wf, yf = (bf16_bits_to_f32(v).astype(np.float64) for v in (x, w, dy))
+    s_f = np.dot(yf, f.cpu().numpy().astype(np.float64))
+    s_x = np.dot(xf, gx.cpu().numpy().astype(np.float64))
+    s_w = np.dot(wf, gw.cpu().numpy().astype(np.float64))
+    assert abs(s_f - s_x) <= 1e-4 * abs(s_f) and abs(s_f - s_w) <= 1e-4 * abs(s_f)

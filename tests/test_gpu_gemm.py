@@ -1,0 +1,192 @@
+"""Batched GEMM on the GPU against the oracle (the reference's accumulation restated on the CPU).
+
+Tolerance: relative Frobenius error of the fp32 accumulators <= 2e-3 for bf16 / fp32 operands and <= 1e-2 for fp8
+operands (the bound the path's specification states); observed errors are orders of magnitude below.
+"""
+import numpy as np
+import pytest
+
+from intel_gaudi3_software_amd import Epilogue, MmeSimTensor, abi
+from helpers import A, TOL, decode_operand, desc, random_operand, rel_frobenius
+
+pytestmark = pytest.mark.gpu
+
+OPS = [abi.OP_AB, abi.OP_ABT, abi.OP_ATB, abi.OP_ATBT]
+TYPES = [(abi.BF16, abi.BF16, 0, 0, 0, 0), (abi.FP32, abi.FP32, 0, 0, 0, 0), (abi.FP8_143, abi.FP8_143, 7, 7, 0, 0),
+         (abi.FP8_143, abi.FP8_152, 7, 15, 0, 0), (abi.FP8_152, abi.FP8_143, 20, 3, 0, 2), (abi.FP8_152, abi.FP8_152, 15, 1, 0, 0)]
+
+
+def _shapes(op, M, N, K):
+    ta = op in (abi.OP_ATB, abi.OP_ATBT)
+    tb = op in (abi.OP_ABT, abi.OP_ATBT)
+    return ([M, K] if ta else [K, M]), ([K, N] if tb else [N, K])
+
+
+def _run_both(calc, orc, op, M, N, K, dtA, dtB, bA, bB, mA, mB, batch=(1, 1, 1), bcast_b=False, seed=0, device=False,
+              pad=(0, 0, 0)):
+    import torch
+    rng = np.random.default_rng(seed)
+    asz, bsz = _shapes(op, M, N, K)
+    nb = int(np.prod(batch))
+    bbatch = (1, 1, 1) if bcast_b else batch
+    nbb = int(np.prod(bbatch))
+    a_ld, b_ld, o_ld = asz[0] + pad[0], bsz[0] + pad[1], N + pad[2]
+    a = random_operand(rng, dtA, a_ld * asz[1] * nb, orc, bA, mA)
+    b = random_operand(rng, dtB, b_ld * bsz[1] * nbb, orc, bB, mB)
+    o_ref = np.zeros(o_ld * M * nb, np.float32)
+    o_gpu = np.zeros(o_ld * M * nb, np.float32)
+    sa, sb, so = ([1, a_ld] if pad[0] else None), ([1, b_ld] if pad[1] else None), ([1, o_ld] if pad[2] else None)
+    da = desc(a, asz + list(batch), dtA, bA, mA, sa)
+    db = desc(b, bsz + list(bbatch), dtB, bB, mB, sb)
+    do = desc(o_ref, [N, M] + list(batch), abi.FP32, strides=so)
+    assert orc.orc_batch_gemm(A(do), A(da), A(db), op) == 0, orc.orc_last_error()
+    if device:
+        tt = {abi.BF16: torch.int16, abi.FP32: torch.float32}
+        ta = torch.from_numpy(a.view(np.int16) if dtA == abi.BF16 else a).cuda()
+        tb = torch.from_numpy(b.view(np.int16) if dtB == abi.BF16 else b).cuda()
+        to = torch.zeros(o_gpu.size, dtype=torch.float32, device="cuda")
+        calc.doBatchGemm(MmeSimTensor([N, M] + list(batch), 5, abi.FP32, to, strides=so),
+                         MmeSimTensor(asz + list(batch), 5, dtA, ta, bA, mA, sa),
+                         MmeSimTensor(bsz + list(bbatch), 5, dtB, tb, bB, mB, sb), op)
+        calc.synchronize()
+        o_gpu = to.cpu().numpy()
+    else:
+        calc.doBatchGemm(MmeSimTensor([N, M] + list(batch), 5, abi.FP32, o_gpu, strides=so),
+                         MmeSimTensor(asz + list(batch), 5, dtA, a, bA, mA, sa),
+                         MmeSimTensor(bsz + list(bbatch), 5, dtB, b, bB, mB, sb), op)
+    return o_gpu, o_ref
+
+
+@pytest.mark.parametrize("dtA,dtB,bA,bB,mA,mB", TYPES)
+@pytest.mark.parametrize("op", OPS)
+def test_gemm_small_ragged(calc, orc, op, dtA, dtB, bA, bB, mA, mB):
+    """Sizes that are multiples of nothing: the element-wise load path, edge tiles, batch with a broadcast operand."""
+    got, want = _run_both(calc, orc, op, 13, 11, 37, dtA, dtB, bA, bB, mA, mB, batch=(2, 3, 1), bcast_b=True, seed=op)
+    assert rel_frobenius(got, want) <= TOL[dtA]
+
+
+@pytest.mark.parametrize("dtA,dtB,bA,bB,mA,mB", TYPES)
+@pytest.mark.parametrize("op", OPS)
+def test_gemm_aligned_vector_path(calc, orc, op, dtA, dtB, bA, bB, mA, mB):
+    """Aligned sizes: 16-byte vector loads, register transposes, several k stages, more than one tile per axis."""
+    got, want = _run_both(calc, orc, op, 160, 144, 208, dtA, dtB, bA, bB, mA, mB, seed=10 + op, device=True)
+    assert rel_frobenius(got, want) <= TOL[dtA]
+
+
+def test_gemm_strided_rows_keep_gaps(calc, orc):
+    """Row pitches larger than the row (sub-views): gaps in the output keep their previous contents."""
+    got, want = _run_both(calc, orc, abi.OP_AB, 9, 10, 20, abi.BF16, abi.BF16, 0, 0, 0, 0, pad=(5, 3, 2), seed=4)
+    assert rel_frobenius(got, want) <= TOL[abi.BF16]
+    # the oracle left the gap columns at 0 (initial value); so must the GPU path
+    gaps = np.ones(got.size, bool).reshape(9, 12)
+    gaps[:, :10] = False
+    assert np.all(got.reshape(9, 12)[gaps] == 0)
+
+
+def test_gemm_config1_bf16_512(calc, orc):
+    """bf16 512^3 -> fp32, seed 1001: the CPU-runnable configuration of the baseline."""
+    got, want = _run_both(calc, orc, abi.OP_AB, 512, 512, 512, abi.BF16, abi.BF16, 0, 0, 0, 0, seed=1001, device=True)
+    err = rel_frobenius(got, want)
+    assert err <= 2e-3
+    # and both agree with the exact product of the decoded operands far inside the tolerance
+    assert err <= 1e-4
+
+
+def test_gemm_zero_common_dim(calc):
+    out = np.full(6, 7.0, np.float32)
+    calc.doBatchGemm(MmeSimTensor([3, 2], 2, abi.FP32, out), MmeSimTensor([0, 2], 2, abi.BF16, np.zeros(4, np.uint16)),
+                     MmeSimTensor([3, 0], 2, abi.BF16, np.zeros(4, np.uint16)), abi.OP_AB)
+    assert np.all(out == 0)
+
+
+def test_fp8_bias_folding_is_exact(calc, orc):
+    """Changing the exponent bias of an operand scales the result by an exact power of two."""
+    import torch
+    rng = np.random.default_rng(21)
+    M = N = K = 64
+    a = rng.integers(0, 0x78, M * K).astype(np.uint8) | (rng.integers(0, 2, M * K).astype(np.uint8) << 7)
+    b = rng.integers(0, 0x78, N * K).astype(np.uint8) | (rng.integers(0, 2, N * K).astype(np.uint8) << 7)
+    res = {}
+    for bias in (3, 7, 11, 15):
+        o = np.zeros(M * N, np.float32)
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, o), MmeSimTensor([K, M], 2, abi.FP8_143, a, bias),
+                         MmeSimTensor([N, K], 2, abi.FP8_143, b, 7), abi.OP_AB)
+        res[bias] = o
+    for bias in (3, 11, 15):
+        assert np.array_equal(res[bias], res[7] * np.float32(2.0 ** (7 - bias)))
+
+
+def test_fp8_special_codes_take_exact_path(calc, orc):
+    """fp8_143 in full inf/nan mode: exponent-15 codes are inf / NaN for Gaudi and finite for the hardware's e4m3.
+    The library must notice them and still agree with the reference (NaN / inf placement included)."""
+    rng = np.random.default_rng(22)
+    M, N, K = 48, 40, 96
+    a = rng.integers(0, 0x70, M * K).astype(np.uint8)
+    b = rng.integers(0, 0x70, N * K).astype(np.uint8)
+    a[5 * K + 3] = 0x78   # +inf in row 5
+    a[9 * K + 1] = 0x7D   # NaN in row 9
+    b[7 * N + 2] = 0xF8   # -inf in column 2 (k = 7)
+    want = np.zeros(M * N, np.float32)
+    da, db, do = desc(a, [K, M], abi.FP8_143, 7), desc(b, [N, K], abi.FP8_143, 7), desc(want, [N, M], abi.FP32)
+    assert orc.orc_batch_gemm(A(do), A(da), A(db), abi.OP_AB) == 0
+    got = np.zeros(M * N, np.float32)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, got), MmeSimTensor([K, M], 2, abi.FP8_143, a, 7),
+                     MmeSimTensor([N, K], 2, abi.FP8_143, b, 7), abi.OP_AB)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.isinf(got), np.isinf(want))
+    fin = np.isfinite(want)
+    assert np.array_equal(np.sign(got[~fin & ~np.isnan(want)]), np.sign(want[~fin & ~np.isnan(want)]))
+    assert rel_frobenius(got[fin], want[fin]) <= 1e-2
+    assert np.isnan(want).any() and np.isinf(want).any()
+
+
+@pytest.mark.parametrize("out_dt,out_bias", [(abi.BF16, 0), (abi.FP8_143, 7), (abi.FP8_152, 15), (abi.FP32, 0)])
+def test_fused_epilogue_equals_gemm_then_cast(calc, orc, out_dt, out_bias):
+    """Fused descale + relu + cast == (fp32 GEMM on the GPU) -> oracle cast of the same accumulators, bit for bit."""
+    import torch
+    rng = np.random.default_rng(31)
+    M, N, K = 96, 80, 128
+    a = random_operand(rng, abi.FP8_143, M * K, orc, 7)
+    b = random_operand(rng, abi.FP8_152, N * K, orc, 15, scale=0.05)
+    col = rng.integers(-3, 4, N).astype(np.int32)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    acc = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    X = MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7)
+    W = MmeSimTensor([N, K], 2, abi.FP8_152, tb, 15)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, acc), X, W, abi.OP_AB)
+    td = {abi.BF16: torch.int16, abi.FP32: torch.float32}.get(out_dt, torch.uint8)
+    out = torch.zeros(M * N, dtype=td, device="cuda")
+    epi = Epilogue(scale_exp=-2, col_scale_exp=torch.from_numpy(col).cuda(), relu=True, clipFp=True)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, out_dt, out, out_bias), X, W, abi.OP_AB, epilogue=epi)
+    calc.synchronize()
+    acc_h = acc.cpu().numpy()
+    want = np.zeros(M * N, abi.DTYPE_NUMPY[out_dt] if out_dt != abi.FP32 else np.uint32)
+    assert orc.orc_cast_from_fp32(want.ctypes.data, out_dt, out_bias, 0, acc_h.ctypes.data, M * N, -2, col.ctypes.data, N, 1,
+                                  0, 1, 0, 0) == 0
+    got = out.cpu().numpy()
+    got = got.view(np.uint16) if out_dt == abi.BF16 else (got.view(np.uint32) if out_dt == abi.FP32 else got)
+    assert np.array_equal(got, want)
+
+
+def test_gemm_linearity_large(calc, orc):
+    """Size-independent property at a large shape (2048 x 1024 x 4096 fp8): doubling A via its exponent bias doubles
+    the result exactly; a 64-row slab agrees with the oracle."""
+    import torch
+    rng = np.random.default_rng(41)
+    M, N, K = 2048, 1024, 4096
+    a = random_operand(rng, abi.FP8_143, M * K, orc, 7, scale=40.0)
+    b = random_operand(rng, abi.FP8_143, N * K, orc, 7, scale=40.0)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    o1 = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    o2 = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, o1), MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7),
+                     MmeSimTensor([N, K], 2, abi.FP8_143, tb, 7), abi.OP_AB)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, o2), MmeSimTensor([K, M], 2, abi.FP8_143, ta, 3),
+                     MmeSimTensor([N, K], 2, abi.FP8_143, tb, 11), abi.OP_AB)
+    calc.synchronize()
+    assert torch.equal(o1, o2)  # 2^(7-3) * 2^(7-11) = 1
+    rows = 64
+    want = np.zeros(rows * N, np.float32)
+    da, db, do = desc(a, [K, rows], abi.FP8_143, 7), desc(b, [N, K], abi.FP8_143, 7), desc(want, [N, rows], abi.FP32)
+    assert orc.orc_batch_gemm(A(do), A(da), A(db), abi.OP_AB) == 0
+    assert rel_frobenius(o1.cpu().numpy()[:rows * N], want) <= 1e-2
