@@ -1,0 +1,56 @@
+"""The C ABI library: it loads, exports every symbol include/mme_hip.h declares, and its argument checks that need no
+device behave like the reference's assertions.  (No compute call is made here.)"""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from intel_gaudi3_software_amd import abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(abi.LIB_PATH):
+        pytest.skip("libmme_hip.so has not been built (python -m intel_gaudi3_software_amd.build)")
+    return abi.load_library()
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mme_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mme_hip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_entry_points():
+    names = _declared()
+    for must in ("mme_hip_create", "mme_hip_destroy", "mme_hip_batch_gemm", "mme_hip_convolution", "mme_hip_activation",
+                 "mme_hip_memory_write", "mme_hip_batch_gemm_dev", "mme_hip_convolution_dev", "mme_hip_cast_from_fp32_dev",
+                 "mme_hip_cast_to_fp32_dev"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    missing = [n for n in _declared() if not hasattr(lib, n)]
+    assert not missing, missing
+    assert b"gfx950" in lib.mme_hip_version()
+
+
+def test_create_rejects_wrong_static_dims_and_chips(lib):
+    h = C.c_void_p()
+    # "dynamic value different than static value" (mme_reference_impl.cpp:143-144): checked before any device is touched
+    assert lib.mme_hip_create(C.byref(h), abi.CHIP_GAUDI3, 4, 4, 0, 256, None, 0) == abi.EINVAL
+    assert b"static value" in lib.mme_hip_last_error(None)
+    assert lib.mme_hip_create(C.byref(h), abi.CHIP_GAUDI2, 5, 4, 0, 256, None, 0) == abi.EUNSUPPORTED
+    assert lib.mme_hip_create(C.byref(h), 17, 5, 4, 0, 256, None, 0) == abi.EINVAL
+    assert not h.value
+
+
+def test_pod_layout_matches_header():
+    # mme_hip_tensor: pointer + 5 + 5 uint32 + 4 int32 ; conv params: 2 + 12 + 1 int32 ; epilogue
+    assert C.sizeof(abi.Tensor) == 8 + 4 * 10 + 4 * 4
+    assert C.sizeof(abi.ConvParams) == 4 * 15
+    assert abi.Tensor.sizes.offset == 8 and abi.Tensor.strides.offset == 28 and abi.Tensor.dim.offset == 48
+    assert C.sizeof(abi.Epilogue) == 40 and abi.Epilogue.col_scale_exp.offset == 8
