@@ -93,42 +93,51 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_from_fp32_kernel(void* __re
     const size_t  n4 = n >> 2;
     const v4f*    in4 = reinterpret_cast<const v4f*>(in);
     OV*           out4 = reinterpret_cast<OV*>(out);
-    const size_t  stride = (size_t) gridDim.x * CAST_THREADS;
-    size_t        i = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x;
-
-    for (; i + (CAST_UNROLL - 1) * stride < n4; i += CAST_UNROLL * stride)
+    // A workgroup owns contiguous chunks of CAST_UNROLL x 256 float4 (16 KiB of input): four fully coalesced 1 KiB
+    // loads per wavefront are issued back to back, then converted and stored.  Streaming (non-temporal) accesses and
+    // one chunk per workgroup measured fastest on MI355X (6.2 TB/s against 4.5 TB/s for a grid-stride loop).
+    constexpr size_t CHUNK = (size_t) CAST_UNROLL * CAST_THREADS;
+    const size_t     n_chunks = (n4 + CHUNK - 1) / CHUNK;
+    for (size_t c = blockIdx.x; c < n_chunks; c += gridDim.x)
     {
-        v4f v[CAST_UNROLL];
-#pragma unroll
-        for (int j = 0; j < CAST_UNROLL; j++) v[j] = __builtin_nontemporal_load(in4 + i + j * stride);
-#pragma unroll
-        for (int j = 0; j < CAST_UNROLL; j++)
+        const size_t i = c * CHUNK + threadIdx.x;
+        if (c * CHUNK + CHUNK <= n4)
         {
-            OV o;
-            if constexpr (COL)
+            v4f v[CAST_UNROLL];
+#pragma unroll
+            for (int j = 0; j < CAST_UNROLL; j++) v[j] = __builtin_nontemporal_load(in4 + i + j * CAST_THREADS);
+#pragma unroll
+            for (int j = 0; j < CAST_UNROLL; j++)
             {
-                const uint32_t c0 = (uint32_t) (((i + j * stride) << 2) % n_cols);
-                const int4     ce = *reinterpret_cast<const int4*>(col_exp + c0);
-                o = cast4<DT, FAST>(v[j], p, v4f {pow2_of(ce.x), pow2_of(ce.y), pow2_of(ce.z), pow2_of(ce.w)});
+                OV o;
+                if constexpr (COL)
+                {
+                    const uint32_t c0 = (uint32_t) (((i + j * CAST_THREADS) << 2) % n_cols);
+                    const int4     ce = *reinterpret_cast<const int4*>(col_exp + c0);
+                    o = cast4<DT, FAST>(v[j], p, v4f {pow2_of(ce.x), pow2_of(ce.y), pow2_of(ce.z), pow2_of(ce.w)});
+                }
+                else
+                    o = cast4<DT, FAST>(v[j], p);
+                __builtin_nontemporal_store(o, out4 + i + j * CAST_THREADS);
             }
-            else
-                o = cast4<DT, FAST>(v[j], p);
-            __builtin_nontemporal_store(o, out4 + i + j * stride);
-        }
-    }
-    for (; i < n4; i += stride)
-    {
-        const v4f v = in4[i];
-        OV        o;
-        if constexpr (COL)
-        {
-            const uint32_t c0 = (uint32_t) ((i << 2) % n_cols);
-            const int4     ce = *reinterpret_cast<const int4*>(col_exp + c0);
-            o = cast4<DT, FAST>(v, p, v4f {pow2_of(ce.x), pow2_of(ce.y), pow2_of(ce.z), pow2_of(ce.w)});
         }
         else
-            o = cast4<DT, FAST>(v, p);
-        out4[i] = o;
+        {
+            for (size_t k = i; k < n4; k += CAST_THREADS)
+            {
+                const v4f v = in4[k];
+                OV        o;
+                if constexpr (COL)
+                {
+                    const uint32_t c0 = (uint32_t) ((k << 2) % n_cols);
+                    const int4     ce = *reinterpret_cast<const int4*>(col_exp + c0);
+                    o = cast4<DT, FAST>(v, p, v4f {pow2_of(ce.x), pow2_of(ce.y), pow2_of(ce.z), pow2_of(ce.w)});
+                }
+                else
+                    o = cast4<DT, FAST>(v, p);
+                out4[k] = o;
+            }
+        }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 3))
     {
@@ -187,37 +196,62 @@ __global__ __launch_bounds__(CAST_THREADS) void cast_to_fp32_kernel(float* __res
     size_t       done = 0;
     if (vec_ok)
     {
-        // four elements per lane and step: one 4 B (fp8) / 8 B (bf16) load, one 16 B store
-        const size_t n4 = n >> 2;
-        float4*      out4 = reinterpret_cast<float4*>(out);
-        for (size_t i = t; i < n4; i += stride)
+        // four elements per lane and step: one 4 B (fp8) / 8 B (bf16) load, one 16 B streaming store; a workgroup owns
+        // contiguous chunks of 4 x 256 such groups
+        const size_t     n4 = n >> 2;
+        v4f*             out4 = reinterpret_cast<v4f*>(out);
+        constexpr size_t CHUNK = (size_t) CAST_UNROLL * CAST_THREADS;
+        const size_t     n_chunks = (n4 + CHUNK - 1) / CHUNK;
+        for (size_t ch = blockIdx.x; ch < n_chunks; ch += gridDim.x)
         {
-            uint32_t c[4];
-            if constexpr (DT == DT_BF16)
-            {
-                const uint2 r = reinterpret_cast<const uint2*>(in)[i];
-                c[0] = r.x & 0xFFFFu;
-                c[1] = r.x >> 16;
-                c[2] = r.y & 0xFFFFu;
-                c[3] = r.y >> 16;
-            }
-            else
-            {
-                const uint32_t r = reinterpret_cast<const uint32_t*>(in)[i];
-                c[0] = r & 0xFFu;
-                c[1] = (r >> 8) & 0xFFu;
-                c[2] = (r >> 16) & 0xFFu;
-                c[3] = r >> 24;
-            }
-            float f[4];
+            uint32_t raw[CAST_UNROLL][2];
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+            for (int u = 0; u < CAST_UNROLL; u++)
             {
-                f[j] = decode1<DT>(c[j], bias, mode);
-                if (has_scale) f[j] *= scale;
-                if (col_exp) f[j] *= pow2_of(col_exp[((i << 2) + j) % n_cols]);
+                const size_t i = ch * CHUNK + threadIdx.x + (size_t) u * CAST_THREADS;
+                raw[u][0] = raw[u][1] = 0;
+                if (i < n4)
+                {
+                    if constexpr (DT == DT_BF16)
+                    {
+                        const v2u r = __builtin_nontemporal_load(reinterpret_cast<const v2u*>(in) + i);
+                        raw[u][0] = r.x;
+                        raw[u][1] = r.y;
+                    }
+                    else
+                        raw[u][0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(in) + i);
+                }
             }
-            out4[i] = make_float4(f[0], f[1], f[2], f[3]);
+#pragma unroll
+            for (int u = 0; u < CAST_UNROLL; u++)
+            {
+                const size_t i = ch * CHUNK + threadIdx.x + (size_t) u * CAST_THREADS;
+                if (i >= n4) continue;
+                uint32_t c[4];
+                if constexpr (DT == DT_BF16)
+                {
+                    c[0] = raw[u][0] & 0xFFFFu;
+                    c[1] = raw[u][0] >> 16;
+                    c[2] = raw[u][1] & 0xFFFFu;
+                    c[3] = raw[u][1] >> 16;
+                }
+                else
+                {
+                    c[0] = raw[u][0] & 0xFFu;
+                    c[1] = (raw[u][0] >> 8) & 0xFFu;
+                    c[2] = (raw[u][0] >> 16) & 0xFFu;
+                    c[3] = raw[u][0] >> 24;
+                }
+                float f[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                {
+                    f[j] = decode1<DT>(c[j], bias, mode);
+                    if (has_scale) f[j] *= scale;
+                    if (col_exp) f[j] *= pow2_of(col_exp[((i << 2) + j) % n_cols]);
+                }
+                __builtin_nontemporal_store(v4f {f[0], f[1], f[2], f[3]}, out4 + i);
+            }
         }
         done = n4 << 2;
     }
@@ -301,10 +335,10 @@ void launch_cast_dt(void* out, const float* in, size_t n, const CastParams& p, c
                     hipStream_t s)
 {
     const bool aligned = (((uintptr_t) out | (uintptr_t) in) & 15u) == 0;
-    // 2048 blocks x 256 lanes x 4 float4 = 32 MiB of input in flight per sweep: >> 256 CUs, few tail effects
     if (aligned && (!col || ((n_cols & 3u) == 0 && ((uintptr_t) col & 15u) == 0)))
     {
-        const int grid = grid_for((n >> 2) / CAST_UNROLL + 1, 4096);
+        // one 16 KiB chunk per workgroup, up to 2^20 workgroups (a 16 GiB input) before workgroups loop
+        const int grid = grid_for(((n >> 2) / CAST_UNROLL + 1) , 1 << 20);
         if (col)
             hipLaunchKernelGGL((cast_from_fp32_kernel<DT, FAST, true>), dim3(grid), dim3(CAST_THREADS), 0, s, out, in, n, p,
                                col, (uint32_t) n_cols);
@@ -351,7 +385,7 @@ hipError_t launch_cast_to_fp32(float* out, const void* in, int dtype, int bias, 
 {
     if (n == 0) return hipSuccess;
     const int vec_ok = (((uintptr_t) out & 15u) == 0) && (((uintptr_t) in & 7u) == 0);
-    const int grid = grid_for(vec_ok ? (n >> 2) + 1 : n, 8192);
+    const int grid = vec_ok ? grid_for((n >> 2) / CAST_UNROLL + 1, 1 << 20) : grid_for(n, 8192);
     const uint32_t nc = (uint32_t) (n_cols ? n_cols : 1);
     switch (dtype)
     {

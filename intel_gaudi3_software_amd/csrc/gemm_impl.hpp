@@ -347,6 +347,9 @@ __device__ __forceinline__ void store_out(EpilogueRef e, long long idx, float v)
     }
 }
 
+// out-of-line form for kernels whose epilogue is fully unrolled over many accumulators
+__device__ __attribute__((noinline)) void store_out_slow(EpilogueRef e, long long idx, float v) { store_out(e, idx, v); }
+
 __device__ __forceinline__ float pow2_of(int e) { return u2f((uint32_t) (e + 127) << 23); }
 
 // A (f_a, k) x B (f_b, k) -> C[f_a][f_b]

@@ -115,6 +115,7 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     if (p.M <= 0 || p.N <= 0 || nb <= 0) return hipSuccess;
+    if (gemm_fp8_fast_applicable(p)) return launch_gemm_fp8_fast(p, s);
     const int tiles = ((p.M + TILE - 1) / TILE) * ((p.N + TILE - 1) / TILE);
     dim3      grid(tiles, (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
     switch (p.dtype)

@@ -84,6 +84,9 @@ struct GemmProblem
 size_t     gemm_workspace_bytes(const GemmProblem& p);
 int        gemm_pick_split_k(const GemmProblem& p, int num_cus);
 hipError_t launch_gemm(const GemmProblem& p, hipStream_t s);
+// large aligned fp8 problems (gemm_fp8_fast.hip); launch_gemm routes to it when applicable
+bool       gemm_fp8_fast_applicable(const GemmProblem& p);
+hipError_t launch_gemm_fp8_fast(const GemmProblem& p, hipStream_t s);
 
 // flags every exponent-all-ones code of an fp8 buffer (inf / NaN in Gaudi's full mode, finite for the hardware's
 // e4m3): *flag |= 1.  mask_kind 0: any code with all exponent bits set; 1: only 0x7F / 0xFF.

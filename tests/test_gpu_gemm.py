@@ -190,3 +190,63 @@ def test_gemm_linearity_large(calc, orc):
     da, db, do = desc(a, [K, rows], abi.FP8_143, 7), desc(b, [N, K], abi.FP8_143, 7), desc(want, [N, rows], abi.FP32)
     assert orc.orc_batch_gemm(A(do), A(da), A(db), abi.OP_AB) == 0
     assert rel_frobenius(o1.cpu().numpy()[:rows * N], want) <= 1e-2
+
+
+# ---- the large-aligned fp8 kernel (256 x 256 tiles, LDS DMA ring, transposed LDS reads) ---------------------------------
+@pytest.mark.parametrize("dtA,dtB,bA,bB", [(abi.FP8_143, abi.FP8_143, 7, 7), (abi.FP8_143, abi.FP8_152, 7, 15),
+                                           (abi.FP8_152, abi.FP8_143, 15, 11), (abi.FP8_152, abi.FP8_152, 20, 15)])
+@pytest.mark.parametrize("op", [abi.OP_AB, abi.OP_ABT])
+def test_fp8_fast_kernel_vs_oracle(calc, orc, op, dtA, dtB, bA, bB):
+    """Shapes that take the fast path (M, N multiples of 256, K multiple of 128 and >= 384), every fp8 flavour pair,
+    both B layouts, batch of 2 with B broadcast; fp32 accumulators against the oracle."""
+    got, want = _run_both(calc, orc, op, 256, 512, 384, dtA, dtB, bA, bB, 0, 0, batch=(2, 1, 1), bcast_b=True, seed=50 + op,
+                          device=True)
+    assert rel_frobenius(got, want) <= 1e-2
+    assert rel_frobenius(got, want) <= 1e-4  # the reference's truncating tree itself sits ~1e-5 from the exact sums
+
+
+def test_fp8_fast_kernel_every_k_position(calc, orc):
+    """One-hot operands walk a single product through every k position and every tile coordinate: catches any
+    fragment / swizzle / transposed-read mix-up that random data could average out."""
+    import torch
+    M, N, K = 256, 256, 512
+    one = 0x38  # 1.0 in fp8_143 bias 7
+    a = np.zeros((M, K), np.uint8)
+    b = np.zeros((K, N), np.uint8)
+    rng = np.random.default_rng(3)
+    perm_m = rng.permutation(M)
+    for k in range(K):
+        a[perm_m[k % M], k] = one
+        b[k, (k * 7 + 3) % N] = 0x40 if k % 2 else one   # 2.0 / 1.0
+    want = (a == one).astype(np.float64) @ np.where(b == 0x40, 2.0, (b == one) * 1.0)
+    ta, tb = torch.from_numpy(a.ravel()).cuda(), torch.from_numpy(b.ravel()).cuda()
+    out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7),
+                     MmeSimTensor([N, K], 2, abi.FP8_143, tb, 7), abi.OP_AB)
+    calc.synchronize()
+    assert np.array_equal(out.cpu().numpy().reshape(M, N).astype(np.float64), want)
+
+
+def test_fp8_fast_kernel_fused_epilogue_bit_exact(calc, orc):
+    """bf16 / fp8 outputs of the fast kernel == its own fp32 accumulators pushed through the oracle cast."""
+    import torch
+    rng = np.random.default_rng(61)
+    M, N, K = 256, 256, 384
+    a = random_operand(rng, abi.FP8_143, M * K, orc, 7)
+    b = random_operand(rng, abi.FP8_152, N * K, orc, 15, scale=0.05)
+    col = rng.integers(-3, 4, N).astype(np.int32)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    X, W = MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7), MmeSimTensor([N, K], 2, abi.FP8_152, tb, 15)
+    acc = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, acc), X, W, abi.OP_AB)
+    for out_dt, out_bias, td in [(abi.BF16, 0, torch.int16), (abi.FP8_143, 7, torch.uint8)]:
+        out = torch.zeros(M * N, dtype=td, device="cuda")
+        epi = Epilogue(scale_exp=3, col_scale_exp=torch.from_numpy(col).cuda(), relu=True, clipFp=True)
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, out_dt, out, out_bias), X, W, abi.OP_AB, epilogue=epi)
+        calc.synchronize()
+        acc_h = acc.cpu().numpy()
+        want = np.zeros(M * N, abi.DTYPE_NUMPY[out_dt])
+        assert orc.orc_cast_from_fp32(want.ctypes.data, out_dt, out_bias, 0, acc_h.ctypes.data, M * N, 3, col.ctypes.data, N, 1, 0,
+                                      1, 0, 0) == 0
+        got = out.cpu().numpy()
+        assert np.array_equal(got.view(want.dtype), want)
