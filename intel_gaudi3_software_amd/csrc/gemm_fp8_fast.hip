@@ -253,47 +253,117 @@ __global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_val
 
     // ---- epilogue: alpha, per-column power of two, relu, cast, store (same conversion functions as the general kernel).
     // The output-type dispatch sits outside the fully unrolled accumulator walk so that the accumulators stay in
-    // registers; the rare cast settings go through one out-of-line call per element.
+    // registers.  Addresses are a uniform 64-bit tile base plus 32-bit lane offsets (one add per element).
     const long long c_off = b0 * g.epi.batch_stride[0] + b1 * g.epi.batch_stride[1] + b2 * g.epi.batch_stride[2];
     const long long ldc = g.epi.ld;
     const bool      has_alpha = g.epi.has_alpha != 0;
     const float     alpha = g.epi.alpha;
     const int32_t*  col_exp = g.epi.col_exp;
+    const bool      relu = g.epi.fused && g.epi.cast.relu;
+    const int       dt = g.epi.fused ? g.epi.out_dtype : DT_FP32;
+    const int       esz = (dt == DT_FP32) ? 4 : (dt == DT_BF16 ? 2 : 1);
+    char*           tile_base = (char*) g.epi.out + (c_off + (long long) m0 * ldc + n0) * esz; // uniform
+    const uint32_t  ldcb = (uint32_t) ldc * esz;                                              // bytes per output row
+    const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
+                           g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
+    // value of accumulator (i, j, v) after the power-of-two factors and relu
+    auto value = [&](int i, int j, int v, float cs) __attribute__((always_inline))
+    {
+        float x = acc[i][j][v];
+        if (has_alpha) x *= alpha;
+        if (col_exp) x *= cs;
+        if (relu) x = relu_ref(x);
+        return x;
+    };
+    // generic walk: one store per element
     auto walk = [&](auto store) __attribute__((always_inline))
     {
+        const uint32_t lane_off = (uint32_t) (wm * 128 + 4 * (lane >> 5)) * ldcb + (uint32_t) (wn * 128 + (lane & 31)) * esz;
 #pragma unroll
         for (int j = 0; j < 4; j++)
         {
-            const int n = n0 + wn * 128 + j * 32 + (lane & 31);
-            float     cs = 1.0f;
-            if (col_exp) cs = pow2_of(col_exp[n]);
+            float cs = 1.0f;
+            if (col_exp) cs = pow2_of(col_exp[n0 + wn * 128 + j * 32 + (lane & 31)]);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                    store(tile_base + (lane_off + (uint32_t) (i * 32 + 8 * (v >> 2) + (v & 3)) * ldcb + (uint32_t) (j * 32 * esz)), value(i, j, v, cs));
+        }
+    };
+    if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
+        walk([&](char* p, float x) __attribute__((always_inline)) { *(float*) p = x; });
+    else if (dt == DT_BF16 && g.epi.fast_cast)
+    {
+        // bf16, round to nearest even.  Lanes l and l^1 hold neighbouring columns: they swap one packed pair of rows
+        // through DPP so that every lane stores whole dwords (two columns of one row).  NaN, inf and values that round
+        // to inf are rare: a per-tile maximum of |x| detects them and that tile takes the element-wise conversion.
+        const uint32_t odd = lane & 1;
+        const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
+        const uint32_t lane_off = (uint32_t) (wm * 128 + 4 * (lane >> 5) + odd) * ldcb + (uint32_t) (wn * 128 + (lane & 30)) * 2;
+        const uint32_t lane_off1 = (uint32_t) (wm * 128 + 4 * (lane >> 5)) * ldcb + (uint32_t) (wn * 128 + (lane & 31)) * 2;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+        {
+            float cs = 1.0f;
+            if (col_exp) cs = pow2_of(col_exp[n0 + wn * 128 + j * 32 + (lane & 31)]);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+            {
+                uint32_t sum[16], mx = 0;
+#pragma unroll
+                for (int v = 0; v < 16; v++)
+                {
+                    const uint32_t u = f2u(value(i, j, v, cs));
+                    mx = max(mx, u & 0x7FFFFFFFu);
+                    sum[v] = u + 0x7FFFu + ((u >> 16) & 1u); // bf16 code in the high half
+                }
+                if (__builtin_amdgcn_ballot_w64(mx >= 0x7F7F8000u) == 0)
+                {
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2)
+                    {
+                        const uint32_t mine = __builtin_amdgcn_perm(sum[v + 1], sum[v], 0x07060302u); // rows v, v+1 of my column
+                        const uint32_t theirs = (uint32_t) __builtin_amdgcn_update_dpp(0, (int) mine, 0xB1, 0xF, 0xF, false); // lane ^ 1
+                        // even lane: row v = (my col, next col); odd lane: row v+1 = (previous col, my col)
+                        const uint32_t word = __builtin_amdgcn_perm(theirs, mine, sel);
+                        *(uint32_t*) (tile_base + (lane_off + (uint32_t) (i * 32 + 8 * (v >> 2) + (v & 3)) * ldcb + (uint32_t) (j * 64))) = word;
+                    }
+                }
+                else
+                {
+#pragma unroll
+                    for (int v = 0; v < 16; v++)
+                        *(uint16_t*) (tile_base + (lane_off1 + (uint32_t) (i * 32 + 8 * (v >> 2) + (v & 3)) * ldcb + (uint32_t) (j * 64))) =
+                            (uint16_t) fp32_to_bf16_rne(f2u(value(i, j, v, cs)), cp.clip_fp, cp.clip_inf_in);
+                }
+            }
+        }
+    }
+    else if (dt == DT_FP8_143 && g.epi.fast_cast)
+        walk([&](char* p, float x) __attribute__((always_inline)) { *(uint8_t*) p = (uint8_t) fp32_to_fp8_rne_mode0<3>(f2u(x), cp.exp_bias, cp.clip_fp, cp.clip_inf_in); });
+    else if (dt == DT_FP8_152 && g.epi.fast_cast)
+        walk([&](char* p, float x) __attribute__((always_inline)) { *(uint8_t*) p = (uint8_t) fp32_to_fp8_rne_mode0<2>(f2u(x), cp.exp_bias, cp.clip_fp, cp.clip_inf_in); });
+    else
+    {
+        // rare cast settings: element-wise through the out-of-line generic converter (relu is applied there)
+        const uint32_t lane_row = wm * 128 + 4 * (lane >> 5), lane_col = wn * 128 + (lane & 31);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+        {
+            float cs = 1.0f;
+            if (col_exp) cs = pow2_of(col_exp[n0 + lane_col + j * 32]);
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int v = 0; v < 16; v++)
                 {
-                    const int m = m0 + wm * 128 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                    float     x = acc[i][j][v];
+                    float x = acc[i][j][v];
                     if (has_alpha) x *= alpha;
                     if (col_exp) x *= cs;
-                    store(c_off + (long long) m * ldc + n, x);
+                    store_out_slow(g.epi, c_off + (long long) (m0 + lane_row + i * 32 + 8 * (v >> 2) + (v & 3)) * ldc + n0 + lane_col + j * 32, x);
                 }
         }
-    };
-    if (!g.epi.fused) walk([&](long long idx, float x) __attribute__((always_inline)) { ((float*) g.epi.out)[idx] = x; });
-    else
-    {
-        const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
-                               g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
-        const int        dt = g.epi.out_dtype;
-        if (g.epi.fast_cast && dt == DT_BF16)
-            walk([&](long long idx, float x) __attribute__((always_inline)) { ((uint16_t*) g.epi.out)[idx] = (uint16_t) cast_elem<DT_BF16, true>(x, cp); });
-        else if (g.epi.fast_cast && dt == DT_FP8_143)
-            walk([&](long long idx, float x) __attribute__((always_inline)) { ((uint8_t*) g.epi.out)[idx] = (uint8_t) cast_elem<DT_FP8_143, true>(x, cp); });
-        else if (g.epi.fast_cast && dt == DT_FP8_152)
-            walk([&](long long idx, float x) __attribute__((always_inline)) { ((uint8_t*) g.epi.out)[idx] = (uint8_t) cast_elem<DT_FP8_152, true>(x, cp); });
-        else
-            walk([&](long long idx, float x) __attribute__((always_inline)) { store_out_slow(g.epi, idx, x); });
     }
 }
 
@@ -323,6 +393,14 @@ bool gemm_fp8_fast_applicable(const GemmProblem& p)
     if (!p.A.k_contig || !p.A.vec_ok || !p.B.vec_ok) return false;
     if (p.split_k > 1) return false;
     if (p.M % FBM || p.N % FBN || p.K % (2 * FBK) || p.K < 6 * FBK) return false;
+    // epilogue: 32-bit byte offsets inside a tile, dword stores of bf16 pairs
+    if (p.epi.ld <= 0 || p.epi.ld * 4 * FBM >= (1ll << 31)) return false;
+    if (p.epi.fused && p.epi.out_dtype == DT_BF16)
+    {
+        if ((p.epi.ld & 1) || ((uintptr_t) p.epi.out & 3)) return false;
+        for (int d = 0; d < 3; d++)
+            if (p.epi.batch_stride[d] & 1) return false;
+    }
     return true;
 }
 
