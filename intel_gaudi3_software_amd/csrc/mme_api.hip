@@ -564,6 +564,33 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
     const int es = elem_size(A->dtype);
     const int kv = 16 / es;
 
+    if (op == MME_HIP_OP_FWD)
+    {
+        auto dense = [](const mme_hip_tensor* t) {
+            uint64_t acc = 1;
+            for (int d = 0; d < 5; d++)
+            {
+                if (t->sizes[d] > 1 && t->strides[d] != acc) return false;
+                acc *= t->sizes[d];
+            }
+            return ((uintptr_t) t->data % 16) == 0;
+        };
+        const int st[4] = {cp->conv_stride[0], cp->conv_stride[1], cp->conv_stride[2], cp->conv_stride[3]};
+        const int di[4] = {cp->dilation[0], cp->dilation[1], cp->dilation[2], cp->dilation[3]};
+        const int pa[4] = {cp->padding[0], cp->padding[1], cp->padding[2], cp->padding[3]};
+        const bool same = out->sizes[1] == x->sizes[1] && out->sizes[2] == x->sizes[2] && out->sizes[3] == 1 && out->sizes[4] == x->sizes[4];
+        if (same && x->dtype == MME_HIP_BF16 && w->dtype == MME_HIP_BF16 &&
+            conv_fwd_fast_applicable(x->dtype, C, Kc, w->sizes[2], w->sizes[3], w->sizes[4], x->sizes[1], x->sizes[2], x->sizes[3], st, di, pa,
+                                     dense(x) && dense(w) && dense(out)))
+        {
+            GemmEpilogue e;
+            if (int rc = fill_epilogue(h, e, out, epi)) return rc;
+            e.ld = Kc;
+            HIP_TRY(h, launch_conv_fwd_fast(x->data, w->data, x->sizes[4], x->sizes[2], x->sizes[1], e, h->stream));
+            return MME_HIP_OK;
+        }
+    }
+
     GemmProblem g;
     memset(&g, 0, sizeof g);
     g.dtype = A->dtype;

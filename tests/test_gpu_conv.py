@@ -91,3 +91,35 @@ def test_conv_adjoint_identities(calc, orc):
     s_x = np.dot(xf, gx.cpu().numpy().astype(np.float64))
     s_w = np.dot(wf, gw.cpu().numpy().astype(np.float64))
     assert abs(s_f - s_x) <= 1e-4 * abs(s_f) and abs(s_f - s_w) <= 1e-4 * abs(s_f)
+
+
+@pytest.mark.parametrize("B,H,W", [(2, 11, 13), (1, 8, 56), (3, 17, 7)])
+def test_conv_fwd_fast_path_vs_oracle(calc, orc, B, H, W):
+    """The specialised forward kernel (bf16, 3x3, 64 -> 64, stride 1, padding 1): ragged heights / widths, fp32
+    accumulators against the oracle and the fused bf16 output against the oracle cast of the same accumulators."""
+    import torch
+    from intel_gaudi3_software_amd import Epilogue
+    from helpers import to_bf16_bits
+    rng = np.random.default_rng(500 + H)
+    xs, ws, ys = [64, W, H, 1, B], [64, 64, 3, 3, 1], [64, W, H, 1, B]
+    x = to_bf16_bits(np.maximum(rng.standard_normal(int(np.prod(xs))), 0))
+    w = to_bf16_bits(rng.standard_normal(int(np.prod(ws))) * (2.0 / 576) ** 0.5)
+    want = np.zeros(int(np.prod(ys)), np.float32)
+    p = abi.make_conv_params(2, (1, 1, 0), (1, 1, 1), (1, 1, 1))
+    dx, dw, dy = desc(x, xs, abi.BF16), desc(w, ws, abi.BF16), desc(want, ys, abi.FP32)
+    assert orc.orc_convolution(A(dy), A(dx), A(dw), A(dy), A(p), abi.OP_FWD, 0) == 0
+    tx, tw = torch.from_numpy(x.view(np.int16)).cuda(), torch.from_numpy(w.view(np.int16)).cuda()
+    acc = torch.zeros(want.size, dtype=torch.float32, device="cuda")
+    out = torch.zeros(want.size, dtype=torch.int16, device="cuda")
+    X, Wt = MmeSimTensor(xs, 5, abi.BF16, tx), MmeSimTensor(ws, 5, abi.BF16, tw)
+    cp = ConvolutionParams(2, [1, 1, 0, 0], [1, 1, 1, 1], [1, 1, 1, 1])
+    calc.doConvolution(MmeSimTensor(ys, 5, abi.FP32, acc), X, Wt, MmeSimTensor(ys, 5, abi.FP32, acc), cp, abi.OP_FWD)
+    calc.doConvolution(MmeSimTensor(ys, 5, abi.BF16, out), X, Wt, MmeSimTensor(ys, 5, abi.BF16, out), cp, abi.OP_FWD,
+                       epilogue=Epilogue(scale_exp=1, relu=True, clipFp=True))
+    calc.synchronize()
+    got = acc.cpu().numpy()
+    assert rel_frobenius(got, want) <= 2e-3
+    assert rel_frobenius(got, want) <= 1e-4
+    want16 = np.zeros(want.size, np.uint16)
+    assert orc.orc_cast_from_fp32(want16.ctypes.data, abi.BF16, 0, 0, got.ctypes.data, got.size, 1, None, 0, 1, 0, 1, 0, 0) == 0
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want16)
