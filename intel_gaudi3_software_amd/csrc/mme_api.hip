@@ -586,7 +586,7 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
             GemmEpilogue e;
             if (int rc = fill_epilogue(h, e, out, epi)) return rc;
             e.ld = Kc;
-            HIP_TRY(h, launch_conv_fwd_fast(x->data, w->data, x->sizes[4], x->sizes[2], x->sizes[1], e, h->stream));
+            HIP_TRY(h, launch_conv_fwd_fast(x->data, w->data, x->sizes[4], x->sizes[2], x->sizes[1], e, h->num_cus, h->stream));
             return MME_HIP_OK;
         }
     }

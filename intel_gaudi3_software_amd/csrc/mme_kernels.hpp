@@ -91,7 +91,7 @@ hipError_t launch_gemm_fp8_fast(const GemmProblem& p, hipStream_t s);
 // forward convolution fast path (conv_fwd_fast.hip): bf16, 3x3, 64 -> 64 channels, stride 1, padding 1, dense NHWC
 bool       conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int W, int H, int D, const int stride[4], const int dil[4],
                                     const int pad[4], bool dense);
-hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int W, const GemmEpilogue& epi, hipStream_t s);
+hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int W, const GemmEpilogue& epi, int num_cus, hipStream_t s);
 
 // flags every exponent-all-ones code of an fp8 buffer (inf / NaN in Gaudi's full mode, finite for the hardware's
 // e4m3): *flag |= 1.  mask_kind 0: any code with all exponent bits set; 1: only 0x7F / 0xFF.
