@@ -32,10 +32,16 @@ namespace
 constexpr int CF_C = 64, CF_K = 64, CF_TAPS = 9, CF_TR = 4;
 constexpr int CF_WT_ROW = CF_TAPS * CF_C * 2; // bytes per output-channel row of the transposed filter
 constexpr int CF_WT_BYTES = CF_K * CF_WT_ROW; // 73728
-constexpr int CF_MAX_W = 56;                  // two halo tiles of 6 x (W + 2) x 128 B next to the filter in 160 KiB
 constexpr int CF_MAX_DMA = 11;                // DMA requests per wavefront and tile: ceil(6 * 58 * 8 / 64 / 4)
+constexpr int CF_MAX_W = 56;                  // two halo tiles of 6 x (W + 2) x 128 B next to the filter in 160 KiB
 
 __device__ __attribute__((aligned(16))) uint32_t cf_zero_page[4];
+#ifdef CF_EXP_TIMING
+__device__ long long cf_tbuf[256 * 32];
+#define CF_STAMP(i) do { if (tid == 0) cf_tbuf[blockIdx.x * 32 + (i)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define CF_STAMP(i) do { } while (0)
+#endif
 
 struct ConvFwdFastArgs
 {
@@ -52,13 +58,25 @@ __device__ __forceinline__ void cf_dma16(const void* g, uint32_t lds_off)
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_off) : "memory");
 }
 
+// the same with the global address given as a wave-uniform base plus a 32-bit byte offset per lane
+__device__ __forceinline__ void cf_dma16_off(const void* base, uint32_t off, uint32_t lds_off)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds_off) : "memory");
+}
+
 typedef float    cf_v4f __attribute__((ext_vector_type(4)));
 typedef uint32_t cf_v4u __attribute__((ext_vector_type(4)));
+typedef float    cf_v2f __attribute__((ext_vector_type(2)));
+typedef __bf16   cf_v2bf __attribute__((ext_vector_type(2)));
+
+typedef short cf_v4s __attribute__((ext_vector_type(4)));
+#define CF_LDS __attribute__((address_space(3)))
 
 union CfFrag
 {
-    uint4 u;
-    v8bf  v;
+    uint4  u;
+    v8bf   v;
+    cf_v4s h[2];
 };
 
 __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by_value)
@@ -69,67 +87,103 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    CF_STAMP(0);
+#ifdef CF_EXP_TIMING
+    if (tid == 0) cf_tbuf[blockIdx.x * 32 + 30] = wall_clock64();
+#endif
     const int H = a.H, W = a.W, wp = W + 2;
-    const int row_tiles = (H + CF_TR - 1) / CF_TR;
-    const int units = a.B * row_tiles;
-    const int u_begin = (int) ((long long) blockIdx.x * units / gridDim.x), u_end = (int) ((long long) (blockIdx.x + 1) * units / gridDim.x);
-    const int halo_chunks = (CF_TR + 2) * wp * 8;       // 16-byte chunks of one halo tile
-    const int halo_bytes = halo_chunks * 16;
-    const uint32_t lds_base = (uint32_t) (uintptr_t) lds; // LDS byte address of the dynamic segment
-    char*          wt = lds;
-    const uint32_t halo_base = CF_WT_BYTES;
+    // this workgroup's run of output rows (row index = image * H + row); a unit is up to 4 of them inside one image
+    const long long rows_total = (long long) a.B * H;
+    const int       row_begin = (int) (blockIdx.x * rows_total / gridDim.x), row_end = (int) ((blockIdx.x + 1) * rows_total / gridDim.x);
+    const int       halo_bytes = (CF_TR + 2) * wp * 128;
+    const uint32_t  lds_base = (uint32_t) (uintptr_t) lds; // LDS byte address of the dynamic segment
+    const char*     wt = lds;
+    const uint32_t  halo_base = CF_WT_BYTES;
 
-    // ---- DMA plan of one halo tile: this lane's chunk in each of the wavefront's requests ------------------------------
-    // LDS chunk q = (row * wp + col) * 8 + j holds input channels 8 * (j ^ ((col >> 1) & 7)) .. + 7 of halo pixel (row, col)
-    int dma_rel[CF_MAX_DMA]; // element offset from the unit's first input pixel (row h0, column 0); INT_MIN: column outside
-    int dma_row[CF_MAX_DMA]; // halo row 0 .. 5, -1: no chunk (tail of the last request)
+    // ---- input tile with halo by DMA: request i moves LDS chunks 64 * i .. 64 * i + 63, one per lane; wavefront w issues
+    // requests w, w + 4, ...  LDS chunk q = (row * wp + col) * 8 + j holds input channels 8 * (j ^ ((col >> 1) & 7)) .. + 7
+    // of halo pixel (row, col) --------------------------------------------------------------------------------------------
+    int dma_rel[CF_MAX_DMA]; // byte offset from the input pixel (row h0 - 1, column 0) of the unit; -1: no chunk to fetch
+    int dma_row[CF_MAX_DMA]; // halo row 0 .. 5 (beyond: no such chunk)
 #pragma unroll
     for (int j = 0; j < CF_MAX_DMA; j++)
     {
         const int q = (wave + 4 * j) * 64 + lane;
         const int pix = q >> 3, row = pix / wp, col = pix - row * wp;
         const int chunk = (q & 7) ^ ((col >> 1) & 7);
-        dma_row[j] = q < halo_chunks ? row : -1;
-        dma_rel[j] = (col >= 1 && col <= W) ? ((row - 1) * W + (col - 1)) * CF_C + chunk * 8 : INT_MIN;
+        dma_row[j] = row;
+        dma_rel[j] = (col >= 1 && col <= W && row < CF_TR + 2) ? ((row * W + (col - 1)) * CF_C + chunk * 8) * 2 : -1;
     }
-    auto issue_halo = [&](int u, int buf) __attribute__((always_inline))
+    // the halo columns are never fetched: they are zeroed here once, in both tiles
+    for (int i = tid; i < 2 * (CF_TR + 2) * 2 * 8; i += 256)
     {
-        const int       img = u / row_tiles, h0 = (u - img * row_tiles) * CF_TR;
-        const uint16_t* org = a.x + ((size_t) img * H + h0) * W * CF_C;
-#pragma unroll
-        for (int j = 0; j < CF_MAX_DMA; j++)
-        {
-            const int   h = h0 - 1 + dma_row[j];
-            const bool  inside = dma_rel[j] != INT_MIN && h >= 0 && h < H;
-            const void* src = inside ? (const void*) (org + dma_rel[j]) : (const void*) cf_zero_page;
-            if (dma_row[j] >= 0) cf_dma16(src, lds_base + halo_base + buf * halo_bytes + (wave + 4 * j) * 1024);
-        }
+        const int chunk = i & 7, side = (i >> 3) & 1, row = (i >> 4) % (CF_TR + 2), b = (i >> 4) / (CF_TR + 2);
+        *reinterpret_cast<uint4*>(lds + halo_base + b * halo_bytes + ((row * wp + (side ? W + 1 : 0)) * 8 + chunk) * 16) = make_uint4(0, 0, 0, 0);
+    }
+    // org = input pixel (row h0_ - 1, column 0) of the image.  A unit whose six halo rows all lie inside the image
+    // fetches them all (also those a short unit does not need) with one address add per request; a unit at the upper
+    // or lower border fetches the missing rows from a page of zeros
+    auto issue_interior = [&](int j, const uint16_t* org, int buf_) __attribute__((always_inline))
+    {
+        if (dma_rel[j] >= 0) cf_dma16_off(org, (uint32_t) dma_rel[j], lds_base + halo_base + buf_ * halo_bytes + (wave + 4 * j) * 1024);
     };
-    if (u_begin < u_end) issue_halo(u_begin, 0);
-
-    // ---- filter: global [tap][c][k] (k contiguous) -> LDS [k][tap * 64 + c]; 8 x 8 blocks transposed in registers ----
-#pragma unroll
-    for (int it = 0; it < 3; it++)
+    auto issue_border = [&](int j, const uint16_t* org, int h0_, int nrows_, int buf_) __attribute__((always_inline))
     {
-        const int blk = tid + it * 256;
-        if (blk < (CF_TAPS * CF_C / 8) * (CF_K / 8))
+        const int   h = h0_ - 1 + dma_row[j];
+        const void* src = (h >= 0 && h < H) ? (const void*) ((const char*) org + dma_rel[j]) : (const void*) cf_zero_page;
+        if (dma_rel[j] >= 0 && dma_row[j] < nrows_ + 2) cf_dma16(src, lds_base + halo_base + buf_ * halo_bytes + (wave + 4 * j) * 1024);
+    };
+    auto is_interior = [&](int h0_) { return h0_ >= 1 && h0_ + CF_TR + 1 <= H; };
+    auto unit_at = [&](int row, int& img, int& h0, int& nrows) __attribute__((always_inline))
+    {
+        img = row / H;
+        h0 = row - img * H;
+        nrows = min(CF_TR, min(H - h0, row_end - row));
+    };
+    int img, h0, nrows;
+    unit_at(row_begin, img, h0, nrows);
+    if (row_begin < row_end)
+    {
+        const uint16_t* org = a.x + ((long long) img * H + h0 - 1) * W * CF_C;
+#pragma unroll
+        for (int j = 0; j < CF_MAX_DMA; j++) issue_border(j, org, h0, nrows, 0);
+    }
+
+    // ---- filter by DMA in its global order: row R = tap * 64 + in channel (128 bytes = 64 out channels), the 32-byte
+    // blocks of a row XOR-swizzled by R & 3 so that the transposing reads below touch every bank once ---------------------
+    {
+        // wavefront w moves the 18 KiB from w * 18 KiB on: one M0 setting serves four requests through the
+        // instruction offset, which advances the global and the LDS address alike
+        const char* src = (const char*) a.w + (((lane & ~7) | ((lane & 7) ^ (((lane >> 3) & 3) << 1))) << 4) + wave * (CF_WT_BYTES / 4);
+        constexpr int PER_WAVE = CF_WT_BYTES / 1024 / 4;
+#pragma unroll
+        for (int k = 0; k < PER_WAVE; k += 4)
         {
-            const int kb = blk & 7, cb = blk >> 3; // cb: block of 8 consecutive (tap, c) rows; kb: block of 8 output channels
-            uint4     in[8], out[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) in[i] = *reinterpret_cast<const uint4*>(a.w + (size_t) (cb * 8 + i) * CF_K + kb * 8);
-            transpose_block<2>(in, out);
-#pragma unroll
-            for (int j = 0; j < 8; j++) *reinterpret_cast<uint4*>(wt + (kb * 8 + j) * CF_WT_ROW + (cb ^ j) * 16) = out[j];
+            const char*    g = src + k * 1024;
+            const uint32_t l = lds_base + wave * (CF_WT_BYTES / 4) + k * 1024;
+            if (k + 4 <= PER_WAVE)
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n\tglobal_load_lds_dwordx4 %0, off offset:1024\n\t"
+                             "global_load_lds_dwordx4 %0, off offset:2048\n\tglobal_load_lds_dwordx4 %0, off offset:3072" ::"v"(g), "s"(l)
+                             : "memory");
+            else
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n\tglobal_load_lds_dwordx4 %0, off offset:1024" ::"v"(g),
+                             "s"(l)
+                             : "memory");
         }
     }
+    CF_STAMP(1);
 
     // ---- per-lane constants of the contraction -------------------------------------------------------------------------
     const int kg = lane >> 5;
-    // filter fragment: row = output channel n * 32 + lane % 32, chunk = tap * 8 + ks * 2 + kg, swizzled by channel & 7
-    int wt_off[4];
+    // filter fragment (matrix-core rows = out channels n * 32 + lane % 32, k = in channels 8 * kg .. + 7 of the k-step):
+    // two ds_read_b64_tr_b16, each handing a lane one out channel of 4 consecutive filter rows; within a group of 16
+    // lanes, lane j addresses the 8-byte piece j % 4 of row j / 4
+    int wl_off[2];
+    {
+        const int g = lane >> 4, j = lane & 15;
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) wt_off[ks] = (lane & 31) * CF_WT_ROW + (((ks * 2 + kg) ^ (lane & 7)) << 4);
+        for (int n = 0; n < 2; n++) wl_off[n] = ((g >> 1) * 8 + (j >> 2)) * 128 + (((n * 2 + (g & 1)) ^ (j >> 2)) << 5) + ((j & 3) << 3);
+    }
     // pixel fragment: this lane's pixel in each of the wavefront's two tiles (clamped into the tile's 4 rows)
     int px_off[2][3][4]; // [tile][s][ks]: byte offset of the chunk in halo row r = 0
 #pragma unroll
@@ -155,18 +209,64 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
     const CastParams cp = {a.epi.cast.dtype,       a.epi.cast.exp_bias, a.epi.cast.inf_nan_mode, a.epi.cast.rm,    a.epi.cast.clip_fp,
                            a.epi.cast.clip_inf_in, a.epi.cast.ftz,      a.epi.cast.relu,         a.epi.cast.scale, a.epi.cast.has_scale};
 
-    for (int u = u_begin; u < u_end; u++)
+    int stores_in_flight = 0; // wave-uniform: 16-byte store instructions issued after the latest DMA requests
+    int buf = 0, unit = 0;
+    for (int row = row_begin; row < row_end; buf ^= 1, unit++)
     {
-        const int buf = (u - u_begin) & 1;
-        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this wavefront's share of the tile has landed
-        __syncthreads();                    // ... and everybody else's; nobody still reads the other buffer
-        if (u + 1 < u_end) issue_halo(u + 1, buf ^ 1);
+        // the DMA requests for this unit were issued before the previous unit's stores, and vector memory operations
+        // retire in issue order: that many stores may still be in flight when the requests have landed
+        if (stores_in_flight == 16) __builtin_amdgcn_s_waitcnt(0x4F70);
+        else if (stores_in_flight == 8)
+            __builtin_amdgcn_s_waitcnt(0x0F78);
+        else if (stores_in_flight == 4)
+            __builtin_amdgcn_s_waitcnt(0x0F74);
+        else
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+        stores_in_flight = 0;
+        CF_STAMP(2 + 4 * unit);
+        __syncthreads(); // the tile (and the filter) is in LDS for everybody; nobody still reads the other buffer
+        CF_STAMP(3 + 4 * unit);
+        // the next unit's tile: its requests are issued between the matrix-core instructions below
+        const bool      more_units = row + nrows < row_end;
+        int             img1 = 0, h1 = 0, nrows1 = 0;
+        if (more_units)
+        {
+            h1 = h0 + nrows;
+            img1 = img;
+            if (h1 >= H)
+            {
+                h1 = 0;
+                img1++;
+            }
+            nrows1 = min(CF_TR, min(H - h1, row_end - row - nrows));
+        }
+        const uint16_t* org1 = a.x + ((long long) img1 * H + h1 - 1) * W * CF_C;
+        // 0: no next unit, 1: all six halo rows of the next unit lie inside its image, 2: next unit at an image border
+        const int prefetch_kind = !more_units ? 0 : is_interior(h1) ? 1 : 2;
+        auto      prefetch = [&](auto kind_c, int j) __attribute__((always_inline))
+        {
+            constexpr int KIND = decltype(kind_c)::value;
+            if (KIND == 1) issue_interior(j, org1, buf ^ 1);
+            if (KIND == 2) issue_border(j, org1, h1, nrows1, buf ^ 1);
+        };
 
-        const int   img = u / row_tiles, h0 = (u - img * row_tiles) * CF_TR;
-        const int   npix = min(CF_TR, H - h0) * W, ntiles = (npix + 31) >> 5;
+        const int   npix = nrows * W, ntiles = (npix + 31) >> 5;
         const char* halo = lds + halo_base + buf * halo_bytes;
         const bool  two = wave + 4 < ntiles;
-        if (wave >= ntiles) continue;
+        if (wave >= ntiles)
+        {
+            if (more_units)
+            {
+#pragma unroll
+                for (int j = 0; j < CF_MAX_DMA; j++) prefetch(std::integral_constant<int, 2>(), j);
+            }
+            row += nrows;
+            img = img1;
+            h0 = h1;
+            nrows = nrows1;
+            continue;
+        }
+        stores_in_flight = !fused ? (two ? 16 : 8) : bf16_fast ? (two ? 8 : 4) : 0;
 
         v16f acc[2][2];
 #pragma unroll
@@ -178,14 +278,17 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
 
         // k-steps 0 .. 35 = (tap, 16 input channels); the fragments of step i + 1 are fetched between the matrix-core
         // instructions of step i (the scheduling barriers pin that order, the compiler derives the LDS waits from it)
-        auto contract = [&](auto nt_c) __attribute__((always_inline))
+        auto contract = [&](auto nt_c, auto kind_c) __attribute__((always_inline))
         {
             constexpr int NT = decltype(nt_c)::value;
-            CfFrag        fw[2][2], fx[2][2];
+            constexpr int NS = CF_TAPS * 4, AHEAD = 2, RING = AHEAD + 1;
+            CfFrag        fw[RING][2], fx[RING][2];
             auto ld_w = [&](int slot, int n, int step) __attribute__((always_inline))
             {
-                const int tap = step >> 2, ks = step & 3;
-                fw[slot][n].u = *reinterpret_cast<const uint4*>(wt + wt_off[ks] + n * 32 * CF_WT_ROW + tap * 128);
+                const int   tap = step >> 2, ks = step & 3;
+                const char* p = wt + wl_off[n] + tap * 8192 + ks * 2048;
+                fw[slot][n].h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((CF_LDS cf_v4s*) p);
+                fw[slot][n].h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((CF_LDS cf_v4s*) (p + 512));
             };
             auto ld_x = [&](int slot, int t, int step) __attribute__((always_inline))
             {
@@ -196,103 +299,180 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
             {
                 acc[t][n] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[slot][n].v, fx[slot][t].v, acc[t][n], 0, 0, 0);
             };
-            ld_w(0, 0, 0);
-            ld_x(0, 0, 0);
-            ld_w(0, 1, 0);
-            if (NT == 2) ld_x(0, 1, 0);
 #pragma unroll
-            for (int step = 0; step < CF_TAPS * 4; step++)
+            for (int step = 0; step < AHEAD; step++)
             {
-                const int  cur = step & 1, nxt = cur ^ 1;
-                const bool more = step + 1 < CF_TAPS * 4;
+                ld_w(step, 0, step);
+                ld_x(step, 0, step);
+                ld_w(step, 1, step);
+                if (NT == 2) ld_x(step, 1, step);
+            }
+#pragma unroll
+            for (int step = 0; step < NS; step++)
+            {
+                const int  cur = step % RING, nxt = (step + AHEAD) % RING;
+                const bool more = step + AHEAD < NS;
+                if (step % 3 == 1 && step / 3 < CF_MAX_DMA) prefetch(kind_c, step / 3);
                 if constexpr (NT == 2)
                 {
-                    if (more) ld_w(nxt, 0, step + 1);
+                    if (more) ld_w(nxt, 0, step + AHEAD);
                     mm(cur, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (more) ld_x(nxt, 0, step + 1);
+                    if (more) ld_x(nxt, 0, step + AHEAD);
                     mm(cur, 0, 1);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (more) ld_w(nxt, 1, step + 1);
+                    if (more) ld_w(nxt, 1, step + AHEAD);
                     mm(cur, 1, 0);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (more) ld_x(nxt, 1, step + 1);
+                    if (more) ld_x(nxt, 1, step + AHEAD);
                     mm(cur, 1, 1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
                 else
                 {
-                    if (more) ld_w(nxt, 0, step + 1);
-                    if (more) ld_x(nxt, 0, step + 1);
+                    if (more) ld_w(nxt, 0, step + AHEAD);
+                    if (more) ld_x(nxt, 0, step + AHEAD);
                     mm(cur, 0, 0);
                     __builtin_amdgcn_sched_barrier(0);
-                    if (more) ld_w(nxt, 1, step + 1);
+                    if (more) ld_w(nxt, 1, step + AHEAD);
                     mm(cur, 0, 1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
         };
-        if (two) contract(std::integral_constant<int, 2>());
+        auto contract_nt = [&](auto nt_c) __attribute__((always_inline))
+        {
+            if (prefetch_kind == 1) contract(nt_c, std::integral_constant<int, 1>());
+            else if (prefetch_kind == 2)
+                contract(nt_c, std::integral_constant<int, 2>());
+            else
+                contract(nt_c, std::integral_constant<int, 0>());
+        };
+        if (two) contract_nt(std::integral_constant<int, 2>());
         else
-            contract(std::integral_constant<int, 1>());
+            contract_nt(std::integral_constant<int, 1>());
 
+        CF_STAMP(4 + 4 * unit);
         // ---- epilogue: accumulator register v of lane l = channel n * 32 + 8 * (v / 4) + 4 * (l / 32) + v % 4 of pixel l % 32 --
         const long long unit_base = ((long long) img * H + h0) * W * CF_K; // element offset of the unit's first output pixel
-#pragma unroll
-        for (int t = 0; t < 2; t++)
+        // one accumulator tile -> 16 consecutive channels of this lane's pixel, scaled
+        auto gather = [&](int t, int n, float (&val)[16]) __attribute__((always_inline))
         {
-            if (t == 1 && !two) break;
-            const int  p = (wave + 4 * t) * 32 + (lane & 31);
-            const bool live = p < npix;
 #pragma unroll
-            for (int n = 0; n < 2; n++)
+            for (int g = 0; g < 2; g++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                {
+                    const float lo = acc[t][n][4 * g + i], hi = acc[t][n][8 + 4 * g + i];
+                    const auto  sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                    val[8 * g + i] = __uint_as_float(sw[0]);
+                    val[8 * g + 4 + i] = __uint_as_float(sw[1]);
+                }
+            if (has_alpha)
             {
-                // after the exchange the lane holds channels n * 32 + kg * 16 + 0 .. 15 of its pixel, in order
-                float val[16];
 #pragma unroll
-                for (int g = 0; g < 2; g++)
+                for (int c = 0; c < 16; c++) val[c] *= alpha;
+            }
+            if (col_exp)
+            {
 #pragma unroll
-                    for (int i = 0; i < 4; i++)
+                for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[n * 32 + kg * 16 + c]);
+            }
+        };
+        // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN (checked
+        // over all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x|
+        // over the lane's 16 values detects them and that tile takes the element-wise conversion
+        auto store_bf16 = [&](auto relu_c) __attribute__((always_inline))
+        {
+            constexpr bool RELU = decltype(relu_c)::value;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+            {
+                if (t == 1 && !two) break;
+                const int p = (wave + 4 * t) * 32 + (lane & 31);
+#pragma unroll
+                for (int n = 0; n < 2; n++)
+                {
+                    float val[16];
+                    gather(t, n, val);
+                    float sum = 0.0f;
+#pragma unroll
+                    for (int c = 0; c < 16; c++)
                     {
-                        const float lo = acc[t][n][4 * g + i], hi = acc[t][n][8 + 4 * g + i];
-                        const auto  sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
-                        val[8 * g + i] = __uint_as_float(sw[0]);
-                        val[8 * g + 4 + i] = __uint_as_float(sw[1]);
+                        if (RELU) val[c] = relu_ref(val[c]);
+                        sum += __builtin_fabsf(val[c]);
                     }
-                const int ch0 = n * 32 + kg * 16;
-#pragma unroll
-                for (int c = 0; c < 16; c++)
-                {
-                    if (has_alpha) val[c] *= alpha;
-                    if (col_exp) val[c] *= pow2_of(col_exp[ch0 + c]);
-                }
-                if (!live) continue;
-                const long long idx = unit_base + (long long) p * CF_K + ch0;
-                if (!fused)
-                {
-                    cf_v4f* o = (cf_v4f*) ((float*) a.epi.out + idx);
-#pragma unroll
-                    for (int c = 0; c < 4; c++) o[c] = cf_v4f {val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3]};
-                }
-                else if (bf16_fast)
-                {
                     uint32_t pk[8];
+                    if (__builtin_amdgcn_ballot_w64(!(sum < 0x1.ffp+127f)) == 0)
+                    {
 #pragma unroll
-                    for (int c = 0; c < 8; c++)
-                        pk[c] = (uint32_t) cast_elem<DT_BF16, true>(val[2 * c], cp) | ((uint32_t) cast_elem<DT_BF16, true>(val[2 * c + 1], cp) << 16);
-                    cf_v4u* o = (cf_v4u*) ((uint16_t*) a.epi.out + idx);
-                    o[0] = cf_v4u {pk[0], pk[1], pk[2], pk[3]};
-                    o[1] = cf_v4u {pk[4], pk[5], pk[6], pk[7]};
+                        for (int c = 0; c < 8; c++)
+                        {
+                            const cf_v2bf h = __builtin_convertvector(cf_v2f {val[2 * c], val[2 * c + 1]}, cf_v2bf);
+                            __builtin_memcpy(&pk[c], &h, 4);
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int c = 0; c < 8; c++)
+                            pk[c] = fp32_to_bf16_rne(f2u(val[2 * c]), cp.clip_fp, cp.clip_inf_in) |
+                                    (fp32_to_bf16_rne(f2u(val[2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
+                    }
+                    if (p < npix)
+                    {
+                        cf_v4u* o = (cf_v4u*) ((uint16_t*) a.epi.out + unit_base + (long long) p * CF_K + n * 32 + kg * 16);
+                        o[0] = cf_v4u {pk[0], pk[1], pk[2], pk[3]};
+                        o[1] = cf_v4u {pk[4], pk[5], pk[6], pk[7]};
+                    }
                 }
-                else
+            }
+        };
+        if (bf16_fast)
+        {
+            if (cp.relu) store_bf16(std::true_type());
+            else
+                store_bf16(std::false_type());
+        }
+        else
+        {
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+            {
+                if (t == 1 && !two) break;
+                const int p = (wave + 4 * t) * 32 + (lane & 31);
+#pragma unroll
+                for (int n = 0; n < 2; n++)
                 {
+                    float val[16];
+                    gather(t, n, val);
+                    if (p >= npix) continue;
+                    const long long idx = unit_base + (long long) p * CF_K + n * 32 + kg * 16;
+                    if (!fused)
+                    {
+                        cf_v4f* o = (cf_v4f*) ((float*) a.epi.out + idx);
+#pragma unroll
+                        for (int c = 0; c < 4; c++) o[c] = cf_v4f {val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3]};
+                    }
+                    else
+                    {
 #pragma unroll 1
-                    for (int c = 0; c < 16; c++) store_out_slow(a.epi, idx + c, val[c]);
+                        for (int c = 0; c < 16; c++) store_out_slow(a.epi, idx + c, val[c]);
+                    }
                 }
             }
         }
+        CF_STAMP(5 + 4 * unit);
+        row += nrows;
+        img = img1;
+        h0 = h1;
+        nrows = nrows1;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
+    CF_STAMP(31);
+#ifdef CF_EXP_TIMING
+    if (tid == 0) cf_tbuf[blockIdx.x * 32 + 29] = wall_clock64();
+#endif
 }
 } // namespace
 
@@ -325,9 +505,9 @@ hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int 
     a.H = H;
     a.W = W;
     a.epi = epi;
-    const long long units = (long long) B * ((H + CF_TR - 1) / CF_TR);
-    if (units > 0x7fffffffLL) return hipErrorInvalidValue;
-    const int grid = (int) std::min<long long>(units, num_cus > 0 ? num_cus : 256);
+    const long long rows = (long long) B * H;
+    if (rows > 0x7fffffffLL) return hipErrorInvalidValue;
+    const int grid = (int) std::min<long long>((rows + CF_TR - 1) / CF_TR, num_cus > 0 ? num_cus : 256);
     hipLaunchKernelGGL(conv_fwd_fast_kernel, dim3(grid), dim3(256), lds_bytes, s, a);
     return hipGetLastError();
 }
