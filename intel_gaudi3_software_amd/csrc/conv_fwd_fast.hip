@@ -6,17 +6,20 @@
 // traffic puts it within a factor of two of both rooflines, so every input pixel is fetched from memory once, every
 // output is written once, and the fetches of the next tile run underneath the matrix-core work of the current one.
 //
-//   grid        persistent: one workgroup per compute unit (256 lanes = 4 wavefronts), each walking a contiguous run
-//               of work units; a unit is 4 output rows x W columns of one image, all 64 output channels
-//   LDS         the whole filter, transposed once per workgroup to Wt[out channel][tap * 64 + in channel] (16-byte
-//               chunks XOR-swizzled by channel), and two input tiles with halo (6 rows x (W + 2) pixels x 64 channels,
-//               16-byte chunks XOR-swizzled by column) filled by global->LDS DMA; pixels outside the image are
-//               fetched from a 16-byte page of zeros
+//   grid        persistent: one workgroup per compute unit (256 lanes = 4 wavefronts), each owning a contiguous run of
+//               output rows (row index = image * H + row) that it walks in units of up to 4 rows of one image
+//   LDS         the whole filter in its global order (row = tap * 64 + in channel, 64 out channels each), fetched once
+//               per workgroup by global->LDS DMA and read with the transposing ds_read_b64_tr_b16; two input tiles
+//               with halo (6 rows x (W + 2) pixels x 64 channels, 16-byte chunks XOR-swizzled by column), also by DMA:
+//               the requests for the next unit are issued between the matrix-core instructions of the current one.
+//               The halo columns are zeroed once; rows outside the image are fetched from a 16-byte page of zeros
 //   wavefront   pixel tiles of 32 (tile = wavefront, wavefront + 4), both 32-channel halves: per k-step of 16 channels
-//               2 filter fragments + 2 pixel fragments feed 4 v_mfma_f32_32x32x16_bf16 (channels on the rows of the
-//               accumulator tile, pixels on its columns, so that a lane ends up with runs of consecutive channels)
+//               2 filter fragments + 2 pixel fragments, fetched two steps ahead, feed 4 v_mfma_f32_32x32x16_bf16
+//               (channels on the rows of the accumulator tile, pixels on its columns, so that a lane ends up with
+//               runs of consecutive channels)
 //   epilogue    v_permlane32_swap gathers 16 consecutive channels of one pixel per lane; power-of-two factor, relu,
-//               cast (same converters as everywhere else), 16-byte stores
+//               cast (v_cvt_pk_bf16_f32 where it equals the reference's conversion, the shared converters
+//               otherwise), 16-byte stores
 //
 // Everything else (other filters, channel counts, strides, dtypes) runs on the general kernel.
 #include "gemm_impl.hpp"
@@ -36,12 +39,6 @@ constexpr int CF_MAX_DMA = 11;                // DMA requests per wavefront and 
 constexpr int CF_MAX_W = 56;                  // two halo tiles of 6 x (W + 2) x 128 B next to the filter in 160 KiB
 
 __device__ __attribute__((aligned(16))) uint32_t cf_zero_page[4];
-#ifdef CF_EXP_TIMING
-__device__ long long cf_tbuf[256 * 32];
-#define CF_STAMP(i) do { if (tid == 0) cf_tbuf[blockIdx.x * 32 + (i)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define CF_STAMP(i) do { } while (0)
-#endif
 
 struct ConvFwdFastArgs
 {
@@ -87,10 +84,6 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    CF_STAMP(0);
-#ifdef CF_EXP_TIMING
-    if (tid == 0) cf_tbuf[blockIdx.x * 32 + 30] = wall_clock64();
-#endif
     const int H = a.H, W = a.W, wp = W + 2;
     // this workgroup's run of output rows (row index = image * H + row); a unit is up to 4 of them inside one image
     const long long rows_total = (long long) a.B * H;
@@ -171,7 +164,6 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                              : "memory");
         }
     }
-    CF_STAMP(1);
 
     // ---- per-lane constants of the contraction -------------------------------------------------------------------------
     const int kg = lane >> 5;
@@ -223,9 +215,7 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
         else
             __builtin_amdgcn_s_waitcnt(0x0F70);
         stores_in_flight = 0;
-        CF_STAMP(2 + 4 * unit);
         __syncthreads(); // the tile (and the filter) is in LDS for everybody; nobody still reads the other buffer
-        CF_STAMP(3 + 4 * unit);
         // the next unit's tile: its requests are issued between the matrix-core instructions below
         const bool      more_units = row + nrows < row_end;
         int             img1 = 0, h1 = 0, nrows1 = 0;
@@ -352,7 +342,6 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
         else
             contract_nt(std::integral_constant<int, 1>());
 
-        CF_STAMP(4 + 4 * unit);
         // ---- epilogue: accumulator register v of lane l = channel n * 32 + 8 * (v / 4) + 4 * (l / 32) + v % 4 of pixel l % 32 --
         const long long unit_base = ((long long) img * H + h0) * W * CF_K; // element offset of the unit's first output pixel
         // one accumulator tile -> 16 consecutive channels of this lane's pixel, scaled
@@ -368,6 +357,9 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                     val[8 * g + i] = __uint_as_float(sw[0]);
                     val[8 * g + 4 + i] = __uint_as_float(sw[1]);
                 }
+        };
+        auto scale = [&](int n, float (&val)[16]) __attribute__((always_inline))
+        {
             if (has_alpha)
             {
 #pragma unroll
@@ -379,60 +371,87 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[n * 32 + kg * 16 + c]);
             }
         };
+        const bool scaled = has_alpha || col_exp != nullptr;
         // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN (checked
         // over all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x|
-        // over the lane's 16 values detects them and that tile takes the element-wise conversion
-        auto store_bf16 = [&](auto relu_c) __attribute__((always_inline))
+        // over a lane's 16 values detects them and the unit is then converted again element by element.  Straight-line
+        // code on purpose: with one wavefront per SIMD only independent instructions hide each other's latency
+        auto store_bf16 = [&](auto relu_c, auto scale_c, auto nt_c) __attribute__((always_inline))
         {
-            constexpr bool RELU = decltype(relu_c)::value;
+            constexpr bool RELU = decltype(relu_c)::value, SCALE = decltype(scale_c)::value;
+            constexpr int  NT = decltype(nt_c)::value;
+            float          val[NT][2][16];
+            uint32_t       pk[NT][2][8];
+            bool           special = false;
 #pragma unroll
-            for (int t = 0; t < 2; t++)
-            {
-                if (t == 1 && !two) break;
-                const int p = (wave + 4 * t) * 32 + (lane & 31);
+            for (int t = 0; t < NT; t++)
 #pragma unroll
                 for (int n = 0; n < 2; n++)
                 {
-                    float val[16];
-                    gather(t, n, val);
-                    float sum = 0.0f;
+                    gather(t, n, val[t][n]);
+                    if (SCALE) scale(n, val[t][n]);
+                    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int c = 0; c < 16; c++)
                     {
-                        if (RELU) val[c] = relu_ref(val[c]);
-                        sum += __builtin_fabsf(val[c]);
+                        if (RELU) val[t][n][c] = relu_ref(val[t][n][c]);
+                        sum[c & 3] += __builtin_fabsf(val[t][n][c]);
                     }
-                    uint32_t pk[8];
-                    if (__builtin_amdgcn_ballot_w64(!(sum < 0x1.ffp+127f)) == 0)
+                    special |= !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
+#pragma unroll
+                    for (int c = 0; c < 8; c++)
                     {
+                        const cf_v2bf h = __builtin_convertvector(cf_v2f {val[t][n][2 * c], val[t][n][2 * c + 1]}, cf_v2bf);
+                        __builtin_memcpy(&pk[t][n][c], &h, 4);
+                    }
+                }
+            if (__builtin_amdgcn_ballot_w64(special) != 0)
+            {
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int n = 0; n < 2; n++)
 #pragma unroll
                         for (int c = 0; c < 8; c++)
-                        {
-                            const cf_v2bf h = __builtin_convertvector(cf_v2f {val[2 * c], val[2 * c + 1]}, cf_v2bf);
-                            __builtin_memcpy(&pk[c], &h, 4);
-                        }
-                    }
-                    else
-                    {
+                            pk[t][n][c] = fp32_to_bf16_rne(f2u(val[t][n][2 * c]), cp.clip_fp, cp.clip_inf_in) |
+                                          (fp32_to_bf16_rne(f2u(val[t][n][2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
+            }
 #pragma unroll
-                        for (int c = 0; c < 8; c++)
-                            pk[c] = fp32_to_bf16_rne(f2u(val[2 * c]), cp.clip_fp, cp.clip_inf_in) |
-                                    (fp32_to_bf16_rne(f2u(val[2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
-                    }
-                    if (p < npix)
+            for (int t = 0; t < NT; t++)
+            {
+                const int p = (wave + 4 * t) * 32 + (lane & 31);
+                if (p < npix)
+                {
+#pragma unroll
+                    for (int n = 0; n < 2; n++)
                     {
                         cf_v4u* o = (cf_v4u*) ((uint16_t*) a.epi.out + unit_base + (long long) p * CF_K + n * 32 + kg * 16);
-                        o[0] = cf_v4u {pk[0], pk[1], pk[2], pk[3]};
-                        o[1] = cf_v4u {pk[4], pk[5], pk[6], pk[7]};
+                        o[0] = cf_v4u {pk[t][n][0], pk[t][n][1], pk[t][n][2], pk[t][n][3]};
+                        o[1] = cf_v4u {pk[t][n][4], pk[t][n][5], pk[t][n][6], pk[t][n][7]};
                     }
                 }
             }
         };
+        auto store_bf16_nt = [&](auto relu_c, auto scale_c) __attribute__((always_inline))
+        {
+            if (two) store_bf16(relu_c, scale_c, std::integral_constant<int, 2>());
+            else
+                store_bf16(relu_c, scale_c, std::integral_constant<int, 1>());
+        };
         if (bf16_fast)
         {
-            if (cp.relu) store_bf16(std::true_type());
+            if (scaled)
+            {
+                if (cp.relu) store_bf16_nt(std::true_type(), std::true_type());
+                else
+                    store_bf16_nt(std::false_type(), std::true_type());
+            }
             else
-                store_bf16(std::false_type());
+            {
+                if (cp.relu) store_bf16_nt(std::true_type(), std::false_type());
+                else
+                    store_bf16_nt(std::false_type(), std::false_type());
+            }
         }
         else
         {
@@ -446,6 +465,7 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 {
                     float val[16];
                     gather(t, n, val);
+                    scale(n, val);
                     if (p >= npix) continue;
                     const long long idx = unit_base + (long long) p * CF_K + n * 32 + kg * 16;
                     if (!fused)
@@ -462,17 +482,12 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 }
             }
         }
-        CF_STAMP(5 + 4 * unit);
         row += nrows;
         img = img1;
         h0 = h1;
         nrows = nrows1;
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);
-    CF_STAMP(31);
-#ifdef CF_EXP_TIMING
-    if (tid == 0) cf_tbuf[blockIdx.x * 32 + 29] = wall_clock64();
-#endif
 }
 } // namespace
 
