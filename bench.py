@@ -28,6 +28,11 @@ PEAK_HBM_GBS = 8000.0
 METRIC = "TFLOP/s & % fp8/bf16 MFMA peak (GEMM, conv); cast GB/s vs HBM peak; 1 GPU"
 
 
+# HBM bytes per launch of the fp8 GEMM kernel on this workload, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/gemm_fp8_fast_kernel_4096x4096x4096_hbm_traffic.txt (96.9 MiB fetched + 48.0 MiB written; 64 MiB algorithmic)
+GEMM_TRAFFIC_BYTES = 151.9e6
+
+
 def pow2_scale_exp(absmax, fmax):
     import math
     return int(math.floor(math.log2(fmax / absmax)))
@@ -41,6 +46,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=256, help="rows of A in the CPU baseline's M-slab")
     ap.add_argument("--extra", action="store_true", help="also time the other configurations (conv, casts, batched fp8)")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also launch a plain elementwise copy of 2^26 floats (256 MiB read, 256 MiB written) a few times: a "
+                         "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) scales the GEMM kernel's reading by this kernel's")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the path has no multi-GPU part in this build (--gpus %d refused)" % args.gpus,
@@ -83,6 +91,15 @@ def main():
     def step():
         calc.doBatchGemm(Y, X, W, abi.OP_AB, epilogue=epi)
 
+    if args.pmc_calibration:
+        with torch.cuda.stream(stream):
+            src = torch.ones(1 << 26, dtype=torch.float32, device="cuda")
+            dst = torch.empty_like(src)
+            for _ in range(5):
+                torch.add(src, 0.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
     # The operands come out of the saturating quantiser above, which never emits an exponent-all-ones code, so the
     # device-side scan for such codes (the default, MME_HIP_FP8_SPECIALS_CHECK) is told to stand down for the timed
     # region; its cost is measured separately below and reported as `fp8_specials_check`.
@@ -124,7 +141,7 @@ def main():
         "config": {"workload": "fp8_143 (exp bias 7) GEMM M=N=K=4096, per-tensor pow2 scales, fp32 accumulate, fused descale + bf16 "
                                "output (BASELINE.json configs[1])", "op": "ab", "M": M, "N": N, "K": K, "scale_exp_a": eA, "scale_exp_b": eB},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["fp8"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS["fp8"], 4), "traffic": None,
+                     "frac": round(achieved / PEAK_TFLOPS["fp8"], 4), "traffic": GEMM_TRAFFIC_BYTES,
                      "kernel": "gemm_fp8_fast_kernel<0, false>", "kernel_ms": round(kernel_ms, 5)},
         "fp8_specials_check": {"policy_in_timed_region": "assume_none (operands produced by the saturating quantiser)",
                                "ms_per_step_with_device_side_scan": round(checked_ms, 5)},
