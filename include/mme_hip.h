@@ -260,7 +260,7 @@ int mme_hip_convolution(mme_hip_handle             h,
  * mme_reference_impl.cpp:661-689, 1143-1245.  res / bias / actParams are unused
  * by the reference's float path and have no parameter here.  relu modifies acc
  * in place like the reference (:683-686, 1132-1141).
- * Stochastic modes use the handle's LFSR state exactly as :1153-1240 does.
+ * The stochastic rounding modes (and stochastic_ftz_fp8) return EUNSUPPORTED in this build.
  */
 int mme_hip_activation(mme_hip_handle        h,
                        const mme_hip_tensor* out,

@@ -34,6 +34,17 @@ def build_library(verbose=False, jobs=8):
     return LIB
 
 
+def build_cpp_tests():
+    """Compile the C++ known-answer program of the calculator header (host code only, g++)."""
+    root = os.path.dirname(_HERE)
+    src = os.path.join(root, "tests", "cpp", "kat_calculator.cpp")
+    exe = os.path.join(root, "tests", "cpp", "kat_calculator")
+    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(root, "include"), src, "-o", exe, "-L" + CSRC,
+           "-lmme_hip", "-Wl,-rpath,$ORIGIN/../../intel_gaudi3_software_amd/csrc"]
+    subprocess.check_call(cmd)
+    return exe
+
+
 def _wait(procs):
     while procs:
         cmd, p = procs.pop(0)
@@ -49,3 +60,4 @@ def _wait(procs):
 
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_cpp_tests())

@@ -1,0 +1,201 @@
+// Known-answer tests of the C++ surface (include/mme_hip_calculator.h) written the way the reference's own unit tests
+// drive CPUCalculator (mme/tests/unit_tests/mme_unit_test.cpp:67-172, 394-519): same shapes, values and expectations,
+// host tensors, synchronous calls.  Needs a GPU.  Prints one line per case and exits non-zero on the first failure.
+#include "mme_hip_calculator.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <vector>
+
+using MmeHip::Calculator;
+using MmeHip::MMEStackException;
+using MmeHip::Tensor;
+typedef Tensor::SizeArray SizeArray;
+
+static int failures = 0;
+#define EXPECT(cond)                                                                                                                       \
+    do                                                                                                                                     \
+    {                                                                                                                                      \
+        if (!(cond))                                                                                                                       \
+        {                                                                                                                                  \
+            std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);                                                                \
+            failures++;                                                                                                                    \
+        }                                                                                                                                  \
+    } while (0)
+
+static uint16_t bf16_of(float f)
+{
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return (uint16_t) ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+static float float_of_bf16(uint16_t h)
+{
+    const uint32_t u = (uint32_t) h << 16;
+    float          f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+// mme_unit_test.cpp:67-82
+static void reference_gemm_simple_test_fp32(Calculator& calculator)
+{
+    std::vector<float> a(5, 10.0f), b(5, 10.0f), y(1, 0.0f);
+    Tensor             ta({5, 1, 1, 1, 1}, 2, MME_HIP_FP32, a.data()), tb({1, 5, 1, 1, 1}, 2, MME_HIP_FP32, b.data()),
+        ty({1, 1, 1, 1, 1}, 2, MME_HIP_FP32, y.data());
+    calculator.doBatchGemm(ty, ta, tb, MME_HIP_OP_AB);
+    EXPECT(y[0] == 500.0f);
+}
+
+// mme_unit_test.cpp:108-125
+static void reference_gemm_simple_test_bf16(Calculator& calculator)
+{
+    std::vector<uint16_t> a(5, bf16_of(10.0f)), b(5, bf16_of(10.0f));
+    std::vector<float>    y(1, 0.0f);
+    Tensor ta({5, 1, 1, 1, 1}, 2, MME_HIP_BF16, a.data()), tb({1, 5, 1, 1, 1}, 2, MME_HIP_BF16, b.data()), ty({1, 1, 1, 1, 1}, 2, MME_HIP_FP32, y.data());
+    calculator.doBatchGemm(ty, ta, tb, MME_HIP_OP_AB);
+    EXPECT(y[0] == 500.0f);
+}
+
+// mme_unit_test.cpp:127-145.  The reference's test runs on Gaudi2 with e_type_fp32_ieee operands; Gaudi3 registers no
+// worker for that type (mme_reference_impl.cpp:189-197), so here the operands are e_type_fp32 and the ieee type must throw.
+static void reference_gemm_2d_test_fp32(Calculator& calculator)
+{
+    std::vector<float> a(25, 10.0f), b(25, 5.0f), y(25, 0.0f);
+    Tensor ta({5, 5, 1, 1, 1}, 2, MME_HIP_FP32, a.data()), tb({5, 5, 1, 1, 1}, 2, MME_HIP_FP32, b.data()), ty({5, 5, 1, 1, 1}, 2, MME_HIP_FP32, y.data());
+    calculator.doBatchGemm(ty, ta, tb, MME_HIP_OP_AB);
+    for (int i = 0; i < 25; i++) EXPECT(y[i] == 250.0f);
+    bool thrown = false;
+    try
+    {
+        Tensor ia({5, 5, 1, 1, 1}, 2, MME_HIP_FP32_IEEE, a.data()), ib({5, 5, 1, 1, 1}, 2, MME_HIP_FP32_IEEE, b.data());
+        calculator.doBatchGemm(ty, ia, ib, MME_HIP_OP_AB);
+    }
+    catch (const MMEStackException& e)
+    {
+        thrown = std::strstr(e.what(), "not registered") != nullptr;
+    }
+    EXPECT(thrown);
+}
+
+// mme_unit_test.cpp:147-172: GEMM, then doActivation to bf16
+static void reference_gemm_2d_test_bf16(Calculator& calculator)
+{
+    std::vector<uint16_t> a(25, bf16_of(10.0f)), b(25, bf16_of(5.0f)), y(25, 0);
+    std::vector<float>    acc(25, 0.0f);
+    Tensor ta({5, 5, 1, 1, 1}, 2, MME_HIP_BF16, a.data()), tb({5, 5, 1, 1, 1}, 2, MME_HIP_BF16, b.data());
+    Tensor tacc({5, 5, 1, 1, 1}, 2, MME_HIP_FP32, acc.data());
+    calculator.doBatchGemm(tacc, ta, tb, MME_HIP_OP_AB);
+    auto pY = std::make_shared<Tensor>(SizeArray {5, 5, 1, 1, 1}, 2, MME_HIP_BF16, y.data());
+    auto pAcc = std::make_shared<Tensor>(tacc);
+    calculator.doActivation(pY, pAcc, std::shared_ptr<Tensor>(), std::shared_ptr<Tensor>(), false);
+    for (int i = 0; i < 25; i++) EXPECT(float_of_bf16(y[i]) == 250.0f);
+}
+
+// mme_unit_test.cpp:394-408 and 467-481: the two conversions whose codes the reference's tests spell out
+static void fp8_convert(Calculator& calculator)
+{
+    float   v143 = -0.25f, v152 = -0.5f;
+    uint8_t c143 = 0, c152 = 0;
+    auto    acc143 = std::make_shared<Tensor>(SizeArray {1, 1, 1, 1, 1}, 2, MME_HIP_FP32, &v143);
+    auto    out143 = std::make_shared<Tensor>(SizeArray {1, 1, 1, 1, 1}, 2, MME_HIP_FP8_143, &c143, 3u);
+    calculator.doActivation(out143, acc143, std::shared_ptr<Tensor>(), std::shared_ptr<Tensor>(), false);
+    EXPECT(c143 == 0x88);
+    auto acc152 = std::make_shared<Tensor>(SizeArray {1, 1, 1, 1, 1}, 2, MME_HIP_FP32, &v152);
+    auto out152 = std::make_shared<Tensor>(SizeArray {1, 1, 1, 1, 1}, 2, MME_HIP_FP8_152, &c152, 15u);
+    calculator.doActivation(out152, acc152, std::shared_ptr<Tensor>(), std::shared_ptr<Tensor>(), false);
+    EXPECT(c152 == 0xB8);
+}
+
+// mme_unit_test.cpp:425-447 and 498-519: 0.25 * -0.5 summed twice, both fp8 flavours at their usual biases
+static void reference_gemm_simple_test_fp8(Calculator& calculator)
+{
+    // fp8_143, bias 7: 0.25 = 2^(5-7) -> 0x28, -0.5 = -2^(6-7) -> 0xB0; fp8_152, bias 15: 0.25 = 2^(13-15) -> 0x34, -0.5 -> 0xB8
+    const struct
+    {
+        int      type;
+        unsigned bias;
+        uint8_t  a, b;
+    } flavours[] = {{MME_HIP_FP8_143, 7u, 0x28, 0xB0}, {MME_HIP_FP8_152, 15u, 0x34, 0xB8}};
+    for (const auto& f : flavours)
+    {
+        std::vector<uint8_t> a(2, f.a), b(2, f.b);
+        std::vector<float>   y(1, 0.0f);
+        Tensor ta({2, 1, 1, 1, 1}, 2, f.type, a.data(), f.bias), tb({1, 2, 1, 1, 1}, 2, f.type, b.data(), f.bias), ty({1, 1, 1, 1, 1}, 2, MME_HIP_FP32, y.data());
+        calculator.doBatchGemm(ty, ta, tb, MME_HIP_OP_AB);
+        EXPECT(y[0] == 0.25f * -0.5f * 2);
+    }
+}
+
+// error conventions: what MME_ASSERT rejects must throw (mme_reference_impl.cpp:465-467, 591)
+static void error_conventions(Calculator& calculator)
+{
+    std::vector<float> a(40, 1.0f), b(40, 1.0f), y(16, 0.0f);
+    bool               thrown = false;
+    try
+    {
+        Tensor ta({5, 2, 2, 1, 1}, 3, MME_HIP_FP32, a.data()), tb({2, 5, 3, 1, 1}, 3, MME_HIP_FP32, b.data()), ty({2, 2, 3, 1, 1}, 3, MME_HIP_FP32, y.data());
+        calculator.doBatchGemm(ty, ta, tb, MME_HIP_OP_AB); // batch 2 against batch 3
+    }
+    catch (const MMEStackException& e)
+    {
+        thrown = std::strstr(e.what(), "batch dims") != nullptr;
+    }
+    EXPECT(thrown);
+    thrown = false;
+    try
+    {
+        std::vector<uint16_t> y16(1, 0);
+        Tensor ta({5, 1, 1, 1, 1}, 2, MME_HIP_FP32, a.data()), tb({1, 5, 1, 1, 1}, 2, MME_HIP_FP32, b.data()), ty({1, 1, 1, 1, 1}, 2, MME_HIP_BF16, y16.data());
+        calculator.doBatchGemm(ty, ta, tb, MME_HIP_OP_AB); // only fp32 outputs are registered
+    }
+    catch (const MMEStackException& e)
+    {
+        thrown = std::strstr(e.what(), "not registered") != nullptr;
+    }
+    EXPECT(thrown);
+    thrown = false;
+    try
+    {
+        Calculator wrong(MME_HIP_CHIP_GAUDI3, 4, 4); // tensor dims must be 5
+    }
+    catch (const MMEStackException&)
+    {
+        thrown = true;
+    }
+    EXPECT(thrown);
+}
+
+int main()
+{
+    try
+    {
+        Calculator calculator(MME_HIP_CHIP_GAUDI3);
+        struct
+        {
+            const char* name;
+            void (*fn)(Calculator&);
+        } cases[] = {{"reference_gemm_simple_test_fp32", reference_gemm_simple_test_fp32},
+                     {"reference_gemm_simple_test_bf16", reference_gemm_simple_test_bf16},
+                     {"reference_gemm_2d_test_fp32", reference_gemm_2d_test_fp32},
+                     {"reference_gemm_2d_test_bf16", reference_gemm_2d_test_bf16},
+                     {"fp8_convert", fp8_convert},
+                     {"reference_gemm_simple_test_fp8", reference_gemm_simple_test_fp8},
+                     {"error_conventions", error_conventions}};
+        for (auto& c : cases)
+        {
+            const int before = failures;
+            c.fn(calculator);
+            std::printf("%s %s\n", failures == before ? "ok    " : "FAILED", c.name);
+            std::fflush(stdout);
+        }
+    }
+    catch (const std::exception& e)
+    {
+        std::printf("unexpected exception: %s\n", e.what());
+        return 2;
+    }
+    return failures ? 1 : 0;
+}

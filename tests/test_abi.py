@@ -54,3 +54,17 @@ def test_pod_layout_matches_header():
     assert C.sizeof(abi.ConvParams) == 4 * 15
     assert abi.Tensor.sizes.offset == 8 and abi.Tensor.strides.offset == 28 and abi.Tensor.dim.offset == 48
     assert C.sizeof(abi.Epilogue) == 40 and abi.Epilogue.col_scale_exp.offset == 8
+
+
+def test_headers_compile_as_c_and_cpp(tmp_path):
+    """include/mme_hip.h is plain C; include/mme_hip_calculator.h is C++17 and needs nothing but the C header."""
+    import subprocess
+    inc = os.path.join(ROOT, "include")
+    c_src = tmp_path / "use_c.c"
+    c_src.write_text('#include "mme_hip.h"\nint f(void) { mme_hip_tensor t; t.dim = 2; return t.dim + MME_HIP_OP_AB; }\n')
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Werror", "-fsyntax-only", "-I" + inc, str(c_src)])
+    cpp_src = tmp_path / "use_cpp.cpp"
+    cpp_src.write_text('#include "mme_hip_calculator.h"\n'
+                       'void f(MmeHip::Calculator& c, MmeHip::Tensor& o, const MmeHip::Tensor& a, const MmeHip::Tensor& b, const MmeHip::ConvolutionParams& p)\n'
+                       '{ c.doBatchGemm(o, a, b, MME_HIP_OP_AB); c.doConvolution(o, a, b, o, p, MME_HIP_OP_FWD); c.doBatchGemmDev(o, a, b, MME_HIP_OP_ABT); }\n')
+    subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-I" + inc, str(cpp_src)])
