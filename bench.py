@@ -234,6 +234,45 @@ def extra_measurements(calc, stream):
     t = timed(lambda: calc.doConvolution(YT, XT, WT, YT, cp, abi.OP_FWD, epilogue=e))
     fl = 2.0 * B * H * Wd * Kk * Cc * 9
     res["conv_fwd_bf16_n64_56x56_c64_k64_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_bf16_peak": fl / t / 1e12 / PEAK_TFLOPS["bf16"]}
+    del tx, tw, ty
+
+    def rand_bf16(n, scale=1.0):
+        return (torch.randn(n, device="cuda") * scale).to(torch.bfloat16).view(torch.int16)
+
+    # c1: bf16 512^3 -> fp32
+    n1 = 512
+    A1, B1 = MmeSimTensor([n1, n1], 2, abi.BF16, rand_bf16(n1 * n1)), MmeSimTensor([n1, n1], 2, abi.BF16, rand_bf16(n1 * n1))
+    Y1 = MmeSimTensor([n1, n1], 2, abi.FP32, torch.zeros(n1 * n1, dtype=torch.float32, device="cuda"))
+    t = timed(lambda: calc.doBatchGemm(Y1, A1, B1, abi.OP_AB))
+    res["gemm_bf16_512x512x512_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n1 ** 3 / t / 1e12, "frac_bf16_peak": 2.0 * n1 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
+    # c4: bf16 3x3 dedx / dedw, N=32 28x28 C=K=256
+    Cc = Kk = 256
+    H = Wd = 28
+    B = 32
+    xs, ws, ys = [Cc, Wd, H, 1, B], [Kk, Cc, 3, 3, 1], [Kk, Wd, H, 1, B]
+    XT = MmeSimTensor(xs, 5, abi.BF16, rand_bf16(int(np.prod(xs))))
+    WT = MmeSimTensor(ws, 5, abi.BF16, rand_bf16(int(np.prod(ws)), 0.02))
+    YT = MmeSimTensor(ys, 5, abi.BF16, rand_bf16(int(np.prod(ys))))
+    DX = MmeSimTensor(xs, 5, abi.FP32, torch.zeros(int(np.prod(xs)), dtype=torch.float32, device="cuda"))
+    DW = MmeSimTensor(ws, 5, abi.FP32, torch.zeros(int(np.prod(ws)), dtype=torch.float32, device="cuda"))
+    fl = 2.0 * B * H * Wd * Kk * Cc * 9
+    t = timed(lambda: calc.doConvolution(DX, XT, WT, YT, cp, abi.OP_DEDX), n=20)
+    res["conv_dedx_bf16_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_bf16_peak": fl / t / 1e12 / PEAK_TFLOPS["bf16"]}
+    t = timed(lambda: calc.doConvolution(DW, XT, WT, YT, cp, abi.OP_DEDW), n=20)
+    res["conv_dedw_bf16_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_bf16_peak": fl / t / 1e12 / PEAK_TFLOPS["bf16"]}
+    del XT, WT, YT, DX, DW
+    # c5: batched mixed fp8: A fp8_143 (bias 7) [4096, 2048, 4] x B fp8_152 (bias 15) [14336, 4096, 1] (broadcast) -> fp8_143
+    M5, K5, N5, b5 = 2048, 4096, 14336, 4
+    qa = torch.randint(0, 0x78, (b5 * M5 * K5,), dtype=torch.uint8, device="cuda")
+    qb = torch.randint(0, 0x7C, (K5 * N5,), dtype=torch.uint8, device="cuda")
+    o5 = torch.zeros(b5 * M5 * N5, dtype=torch.uint8, device="cuda")
+    A5 = MmeSimTensor([K5, M5, b5], 3, abi.FP8_143, qa, 7)
+    B5 = MmeSimTensor([N5, K5, 1], 3, abi.FP8_152, qb, 15)
+    Y5 = MmeSimTensor([N5, M5, b5], 3, abi.FP8_143, o5, 7)
+    e5 = Epilogue(scale_exp=-12, clipFp=True)
+    fl = 2.0 * b5 * M5 * N5 * K5
+    t = timed(lambda: calc.doBatchGemm(Y5, A5, B5, abi.OP_AB, epilogue=e5), n=10, warm=2)
+    res["bgemm_fp8_143x152_4x2048x14336x4096_fp8_out"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
     return res
 
 
