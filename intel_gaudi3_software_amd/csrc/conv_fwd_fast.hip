@@ -6,15 +6,19 @@
 // traffic puts it within a factor of two of both rooflines, so every input pixel is fetched from memory once, every
 // output is written once, and the fetches of the next tile run underneath the matrix-core work of the current one.
 //
-//   grid        persistent: one workgroup per compute unit (256 lanes = 4 wavefronts), each owning a contiguous run of
-//               output rows (row index = image * H + row) that it walks in units of up to 4 rows of one image
+//   grid        persistent: one workgroup of 512 lanes per compute unit, owning a contiguous run of output rows (row
+//               index = image * H + row) cut into units of up to 4 rows of one image.  The 8 wavefronts form two teams
+//               of four (one wavefront of each team per SIMD) that take the units alternately: a wavefront cannot
+//               issue anything else while its own matrix-core instruction occupies it, so the second team's
+//               wavefront on the SIMD is what fills the matrix cores during the first team's loads, stores, waits and
+//               epilogue arithmetic.  Teams synchronise among themselves through counters in LDS, not s_barrier
 //   LDS         the whole filter in its global order (row = tap * 64 + in channel, 64 out channels each), fetched once
-//               per workgroup by global->LDS DMA and read with the transposing ds_read_b64_tr_b16; two input tiles
-//               with halo (6 rows x (W + 2) pixels x 64 channels, 16-byte chunks XOR-swizzled by column), also by DMA:
-//               the requests for the next unit are issued between the matrix-core instructions of the current one.
-//               The halo columns are zeroed once; rows outside the image are fetched from a 16-byte page of zeros
-//   wavefront   pixel tiles of 32 (tile = wavefront, wavefront + 4), both 32-channel halves: per k-step of 16 channels
-//               2 filter fragments + 2 pixel fragments, fetched two steps ahead, feed 4 v_mfma_f32_32x32x16_bf16
+//               per workgroup by global->LDS DMA and read with the transposing ds_read_b64_tr_b16; one input tile with
+//               halo per team (6 rows x (W + 2) pixels x 64 channels, 16-byte chunks XOR-swizzled by column), also by
+//               DMA, requested as soon as the team has finished with its previous tile.  The halo columns are zeroed
+//               once; rows outside the image are fetched from a 16-byte page of zeros
+//   wavefront   pixel tiles of 32 (tile = wavefront in team, + 4), both 32-channel halves: per k-step of 16 channels
+//               2 filter fragments + 2 pixel fragments, fetched one step ahead, feed 4 v_mfma_f32_32x32x16_bf16
 //               (channels on the rows of the accumulator tile, pixels on its columns, so that a lane ends up with
 //               runs of consecutive channels)
 //   epilogue    v_permlane32_swap gathers 16 consecutive channels of one pixel per lane; power-of-two factor, relu,
@@ -45,6 +49,7 @@ struct ConvFwdFastArgs
     const uint16_t* x;   // [B][H][W][64]
     const uint16_t* w;   // [3][3][64 in][64 out]
     int             B, H, W;
+    int             rows_per_wg, rows_extra; // B * H output rows = gridDim.x * rows_per_wg + rows_extra (the first rows_extra workgroups take one more)
     GemmEpilogue    epi; // out = [B][H][W][64], ld = 64
 };
 
@@ -76,7 +81,26 @@ union CfFrag
     cf_v4s h[2];
 };
 
-__global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by_value)
+// n / d for 0 <= n < 2^20, 0 < d < 2^10 without the integer-division sequence: a float estimate, corrected by one
+__device__ __forceinline__ int cf_div(int n, int d)
+{
+    int q = (int) ((float) n * __builtin_amdgcn_rcpf((float) d));
+    const int r = n - q * d;
+    q += (r >= d) - (r < 0);
+    return q;
+}
+
+// Barrier among the four wavefronts of a team: a counter in LDS that only grows.  (s_barrier would stop the other team
+// too.)  Every wavefront of the team reaches every barrier, so the spin always ends.
+__device__ __forceinline__ void cf_team_barrier(uint32_t* counter, uint32_t target, int lane)
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    if (lane == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) __builtin_amdgcn_s_sleep(1);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+__global__ __launch_bounds__(512) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by_value)
 {
     (void) a_by_value;
     typedef const __attribute__((address_space(4))) ConvFwdFastArgs& ArgRef;
@@ -84,84 +108,111 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int team = wave >> 2, tw = wave & 3; // two teams of four wavefronts, one of each team per SIMD
     const int H = a.H, W = a.W, wp = W + 2;
-    // this workgroup's run of output rows (row index = image * H + row); a unit is up to 4 of them inside one image
-    const long long rows_total = (long long) a.B * H;
-    const int       row_begin = (int) (blockIdx.x * rows_total / gridDim.x), row_end = (int) ((blockIdx.x + 1) * rows_total / gridDim.x);
+    // this workgroup's run of output rows (row index = image * H + row); a unit is up to 4 of them inside one image;
+    // the teams take the units of the run alternately
+    const int       row_begin = blockIdx.x * a.rows_per_wg + min((int) blockIdx.x, a.rows_extra);
+    const int       row_end = row_begin + a.rows_per_wg + ((int) blockIdx.x < a.rows_extra ? 1 : 0);
     const int       halo_bytes = (CF_TR + 2) * wp * 128;
     const uint32_t  lds_base = (uint32_t) (uintptr_t) lds; // LDS byte address of the dynamic segment
     const char*     wt = lds;
-    const uint32_t  halo_base = CF_WT_BYTES;
+    const uint32_t  halo_off = CF_WT_BYTES + team * halo_bytes; // this team's input tile
+    const char*     halo = lds + halo_off;
+    uint32_t*       counter = (uint32_t*) (lds + CF_WT_BYTES + 2 * halo_bytes) + team;
+    if (tid < 2) ((uint32_t*) (lds + CF_WT_BYTES + 2 * halo_bytes))[tid] = 0;
 
-    // ---- input tile with halo by DMA: request i moves LDS chunks 64 * i .. 64 * i + 63, one per lane; wavefront w issues
-    // requests w, w + 4, ...  LDS chunk q = (row * wp + col) * 8 + j holds input channels 8 * (j ^ ((col >> 1) & 7)) .. + 7
-    // of halo pixel (row, col) --------------------------------------------------------------------------------------------
+    // ---- input tile with halo by DMA: request i moves LDS chunks 64 * i .. 64 * i + 63, one per lane; wavefront tw of the
+    // team issues requests tw, tw + 4, ...  LDS chunk q = (row * wp + col) * 8 + j holds input channels
+    // 8 * (j ^ ((col >> 1) & 7)) .. + 7 of halo pixel (row, col) ----------------------------------------------------------
     int dma_rel[CF_MAX_DMA]; // byte offset from the input pixel (row h0 - 1, column 0) of the unit; -1: no chunk to fetch
     int dma_row[CF_MAX_DMA]; // halo row 0 .. 5 (beyond: no such chunk)
-#pragma unroll
-    for (int j = 0; j < CF_MAX_DMA; j++)
     {
-        const int q = (wave + 4 * j) * 64 + lane;
-        const int pix = q >> 3, row = pix / wp, col = pix - row * wp;
-        const int chunk = (q & 7) ^ ((col >> 1) & 7);
-        dma_row[j] = row;
-        dma_rel[j] = (col >= 1 && col <= W && row < CF_TR + 2) ? ((row * W + (col - 1)) * CF_C + chunk * 8) * 2 : -1;
+        // request j covers halo pixels 32 j + 8 tw + lane / 8: row and column advance incrementally
+        int row = cf_div(tw * 8 + (lane >> 3), wp), col = tw * 8 + (lane >> 3) - row * wp;
+#pragma unroll
+        for (int j = 0; j < CF_MAX_DMA; j++)
+        {
+            const int chunk = (lane & 7) ^ ((col >> 1) & 7);
+            dma_row[j] = row;
+            dma_rel[j] = (col >= 1 && col <= W && row < CF_TR + 2) ? ((row * W + (col - 1)) * CF_C + chunk * 8) * 2 : -1;
+            col += 32;
+            if (wp >= 32)
+            {
+                const int wrap = col >= wp;
+                col -= wrap ? wp : 0;
+                row += wrap;
+            }
+            else
+            {
+                const int k = cf_div(col, wp);
+                col -= k * wp;
+                row += k;
+            }
+        }
     }
     // the halo columns are never fetched: they are zeroed here once, in both tiles
-    for (int i = tid; i < 2 * (CF_TR + 2) * 2 * 8; i += 256)
+    for (int i = tid; i < 2 * (CF_TR + 2) * 2 * 8; i += 512)
     {
         const int chunk = i & 7, side = (i >> 3) & 1, row = (i >> 4) % (CF_TR + 2), b = (i >> 4) / (CF_TR + 2);
-        *reinterpret_cast<uint4*>(lds + halo_base + b * halo_bytes + ((row * wp + (side ? W + 1 : 0)) * 8 + chunk) * 16) = make_uint4(0, 0, 0, 0);
+        *reinterpret_cast<uint4*>(lds + CF_WT_BYTES + b * halo_bytes + ((row * wp + (side ? W + 1 : 0)) * 8 + chunk) * 16) = make_uint4(0, 0, 0, 0);
     }
-    // org = input pixel (row h0_ - 1, column 0) of the image.  A unit whose six halo rows all lie inside the image
-    // fetches them all (also those a short unit does not need) with one address add per request; a unit at the upper
-    // or lower border fetches the missing rows from a page of zeros
-    auto issue_interior = [&](int j, const uint16_t* org, int buf_) __attribute__((always_inline))
+    // A unit whose six halo rows all lie inside the image fetches them all (also those a short unit does not need) with
+    // one address per request; a unit at the upper or lower border fetches the missing rows from a page of zeros
+    auto issue_halo = [&](int img_, int h0_, int nrows_) __attribute__((always_inline))
     {
-        if (dma_rel[j] >= 0) cf_dma16_off(org, (uint32_t) dma_rel[j], lds_base + halo_base + buf_ * halo_bytes + (wave + 4 * j) * 1024);
+        const uint16_t* org = a.x + ((long long) img_ * H + h0_ - 1) * W * CF_C; // input pixel (row h0_ - 1, column 0)
+        if (h0_ >= 1 && h0_ + CF_TR + 1 <= H)
+        {
+#pragma unroll
+            for (int j = 0; j < CF_MAX_DMA; j++)
+                if (dma_rel[j] >= 0) cf_dma16_off(org, (uint32_t) dma_rel[j], lds_base + halo_off + (tw + 4 * j) * 1024);
+        }
+        else
+        {
+#pragma unroll
+            for (int j = 0; j < CF_MAX_DMA; j++)
+            {
+                const int   h = h0_ - 1 + dma_row[j];
+                const void* src = (h >= 0 && h < H) ? (const void*) ((const char*) org + dma_rel[j]) : (const void*) cf_zero_page;
+                if (dma_rel[j] >= 0 && dma_row[j] < nrows_ + 2) cf_dma16(src, lds_base + halo_off + (tw + 4 * j) * 1024);
+            }
+        }
     };
-    auto issue_border = [&](int j, const uint16_t* org, int h0_, int nrows_, int buf_) __attribute__((always_inline))
+    // the team's current unit; advance() steps to the next unit of the run (one call per unit skipped or done)
+    int  row = row_begin, img = row_begin / H, h0 = row_begin - img * H, nrows = min(CF_TR, min(H - h0, row_end - row_begin));
+    auto advance = [&]() __attribute__((always_inline))
     {
-        const int   h = h0_ - 1 + dma_row[j];
-        const void* src = (h >= 0 && h < H) ? (const void*) ((const char*) org + dma_rel[j]) : (const void*) cf_zero_page;
-        if (dma_rel[j] >= 0 && dma_row[j] < nrows_ + 2) cf_dma16(src, lds_base + halo_base + buf_ * halo_bytes + (wave + 4 * j) * 1024);
-    };
-    auto is_interior = [&](int h0_) { return h0_ >= 1 && h0_ + CF_TR + 1 <= H; };
-    auto unit_at = [&](int row, int& img, int& h0, int& nrows) __attribute__((always_inline))
-    {
-        img = row / H;
-        h0 = row - img * H;
+        row += nrows;
+        h0 += nrows;
+        if (h0 >= H)
+        {
+            h0 = 0;
+            img++;
+        }
         nrows = min(CF_TR, min(H - h0, row_end - row));
     };
-    int img, h0, nrows;
-    unit_at(row_begin, img, h0, nrows);
-    if (row_begin < row_end)
-    {
-        const uint16_t* org = a.x + ((long long) img * H + h0 - 1) * W * CF_C;
-#pragma unroll
-        for (int j = 0; j < CF_MAX_DMA; j++) issue_border(j, org, h0, nrows, 0);
-    }
+    if (team == 1) advance();
+    if (row < row_end) issue_halo(img, h0, nrows);
 
     // ---- filter by DMA in its global order: row R = tap * 64 + in channel (128 bytes = 64 out channels), the 32-byte
-    // blocks of a row XOR-swizzled by R & 3 so that the transposing reads below touch every bank once ---------------------
+    // blocks of a row XOR-swizzled by R & 3 so that the transposing reads below touch every bank once.  Each wavefront
+    // moves 9 KiB; one M0 setting serves four requests through the instruction offset, which advances the global and the
+    // LDS address alike ---------------------------------------------------------------------------------------------------
     {
-        // wavefront w moves the 18 KiB from w * 18 KiB on: one M0 setting serves four requests through the
-        // instruction offset, which advances the global and the LDS address alike
-        const char* src = (const char*) a.w + (((lane & ~7) | ((lane & 7) ^ (((lane >> 3) & 3) << 1))) << 4) + wave * (CF_WT_BYTES / 4);
-        constexpr int PER_WAVE = CF_WT_BYTES / 1024 / 4;
+        constexpr int PER_WAVE = CF_WT_BYTES / 1024 / 8;
+        const char*   src = (const char*) a.w + (((lane & ~7) | ((lane & 7) ^ (((lane >> 3) & 3) << 1))) << 4) + wave * (PER_WAVE * 1024);
 #pragma unroll
         for (int k = 0; k < PER_WAVE; k += 4)
         {
             const char*    g = src + k * 1024;
-            const uint32_t l = lds_base + wave * (CF_WT_BYTES / 4) + k * 1024;
+            const uint32_t l = lds_base + wave * (PER_WAVE * 1024) + k * 1024;
             if (k + 4 <= PER_WAVE)
                 asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n\tglobal_load_lds_dwordx4 %0, off offset:1024\n\t"
                              "global_load_lds_dwordx4 %0, off offset:2048\n\tglobal_load_lds_dwordx4 %0, off offset:3072" ::"v"(g), "s"(l)
                              : "memory");
             else
-                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n\tglobal_load_lds_dwordx4 %0, off offset:1024" ::"v"(g),
-                             "s"(l)
-                             : "memory");
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(l) : "memory");
         }
     }
 
@@ -181,9 +232,9 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
 #pragma unroll
     for (int t = 0; t < 2; t++)
     {
-        int p = (wave + 4 * t) * 32 + (lane & 31);
+        int p = (tw + 4 * t) * 32 + (lane & 31);
         p = min(p, CF_TR * W - 1);
-        const int prow = p / W, pcol = p - prow * W;
+        const int prow = cf_div(p, W), pcol = p - prow * W;
 #pragma unroll
         for (int s = 0; s < 3; s++)
 #pragma unroll
@@ -198,65 +249,38 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
     const int32_t*   col_exp = a.epi.col_exp;
     const int        dt = fused ? a.epi.out_dtype : DT_FP32;
     const bool       bf16_fast = fused && dt == DT_BF16 && a.epi.fast_cast;
+    const bool       scaled = has_alpha || col_exp != nullptr;
     const CastParams cp = {a.epi.cast.dtype,       a.epi.cast.exp_bias, a.epi.cast.inf_nan_mode, a.epi.cast.rm,    a.epi.cast.clip_fp,
                            a.epi.cast.clip_inf_in, a.epi.cast.ftz,      a.epi.cast.relu,         a.epi.cast.scale, a.epi.cast.has_scale};
 
-    int stores_in_flight = 0; // wave-uniform: 16-byte store instructions issued after the latest DMA requests
-    int buf = 0, unit = 0;
-    for (int row = row_begin; row < row_end; buf ^= 1, unit++)
-    {
-        // the DMA requests for this unit were issued before the previous unit's stores, and vector memory operations
-        // retire in issue order: that many stores may still be in flight when the requests have landed
-        if (stores_in_flight == 16) __builtin_amdgcn_s_waitcnt(0x4F70);
-        else if (stores_in_flight == 8)
-            __builtin_amdgcn_s_waitcnt(0x0F78);
-        else if (stores_in_flight == 4)
-            __builtin_amdgcn_s_waitcnt(0x0F74);
-        else
-            __builtin_amdgcn_s_waitcnt(0x0F70);
-        stores_in_flight = 0;
-        __syncthreads(); // the tile (and the filter) is in LDS for everybody; nobody still reads the other buffer
-        // the next unit's tile: its requests are issued between the matrix-core instructions below
-        const bool      more_units = row + nrows < row_end;
-        int             img1 = 0, h1 = 0, nrows1 = 0;
-        if (more_units)
-        {
-            h1 = h0 + nrows;
-            img1 = img;
-            if (h1 >= H)
-            {
-                h1 = 0;
-                img1++;
-            }
-            nrows1 = min(CF_TR, min(H - h1, row_end - row - nrows));
-        }
-        const uint16_t* org1 = a.x + ((long long) img1 * H + h1 - 1) * W * CF_C;
-        // 0: no next unit, 1: all six halo rows of the next unit lie inside its image, 2: next unit at an image border
-        const int prefetch_kind = !more_units ? 0 : is_interior(h1) ? 1 : 2;
-        auto      prefetch = [&](auto kind_c, int j) __attribute__((always_inline))
-        {
-            constexpr int KIND = decltype(kind_c)::value;
-            if (KIND == 1) issue_interior(j, org1, buf ^ 1);
-            if (KIND == 2) issue_border(j, org1, h1, nrows1, buf ^ 1);
-        };
+    // the filter and both teams' first tiles have landed for everybody
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
 
-        const int   npix = nrows * W, ntiles = (npix + 31) >> 5;
-        const char* halo = lds + halo_base + buf * halo_bytes;
-        const bool  two = wave + 4 < ntiles;
-        if (wave >= ntiles)
+    uint32_t barriers = 0;     // team barriers passed so far
+    int      stores_in_flight = 0; // wave-uniform: 16-byte store instructions issued after the latest DMA requests
+    bool     first = true;
+    while (row < row_end)
+    {
+        if (!first)
         {
-            if (more_units)
-            {
-#pragma unroll
-                for (int j = 0; j < CF_MAX_DMA; j++) prefetch(std::integral_constant<int, 2>(), j);
-            }
-            row += nrows;
-            img = img1;
-            h0 = h1;
-            nrows = nrows1;
-            continue;
+            // this wavefront's DMA requests for the unit were issued before the previous unit's stores, and vector memory
+            // operations retire in issue order: that many stores may still be in flight when the requests have landed
+            if (stores_in_flight == 16) __builtin_amdgcn_s_waitcnt(0x4F70);
+            else if (stores_in_flight == 8)
+                __builtin_amdgcn_s_waitcnt(0x0F78);
+            else if (stores_in_flight == 4)
+                __builtin_amdgcn_s_waitcnt(0x0F74);
+            else
+                __builtin_amdgcn_s_waitcnt(0x0F70);
+            cf_team_barrier(counter, 4 * ++barriers, lane); // ... and the other three wavefronts' requests as well
         }
-        stores_in_flight = !fused ? (two ? 16 : 8) : bf16_fast ? (two ? 8 : 4) : 0;
+        first = false;
+        stores_in_flight = 0;
+
+        const int       npix = nrows * W, ntiles = (npix + 31) >> 5;
+        const bool      two = tw + 4 < ntiles;
+        const long long unit_base = ((long long) img * H + h0) * W * CF_K; // element offset of the unit's first output pixel
 
         v16f acc[2][2];
 #pragma unroll
@@ -267,11 +291,12 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 for (int v = 0; v < 16; v++) acc[t][n][v] = 0.0f;
 
         // k-steps 0 .. 35 = (tap, 16 input channels); the fragments of step i + 1 are fetched between the matrix-core
-        // instructions of step i (the scheduling barriers pin that order, the compiler derives the LDS waits from it)
-        auto contract = [&](auto nt_c, auto kind_c) __attribute__((always_inline))
+        // instructions of step i (the scheduling barriers pin that order, the compiler derives the LDS waits from it);
+        // the other team's wavefront on this SIMD fills the issue slots this one leaves open
+        auto contract = [&](auto nt_c) __attribute__((always_inline))
         {
             constexpr int NT = decltype(nt_c)::value;
-            constexpr int NS = CF_TAPS * 4, AHEAD = 2, RING = AHEAD + 1;
+            constexpr int NS = CF_TAPS * 4, AHEAD = 1, RING = AHEAD + 1;
             CfFrag        fw[RING][2], fx[RING][2];
             auto ld_w = [&](int slot, int n, int step) __attribute__((always_inline))
             {
@@ -302,7 +327,6 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
             {
                 const int  cur = step % RING, nxt = (step + AHEAD) % RING;
                 const bool more = step + AHEAD < NS;
-                if (step % 3 == 1 && step / 3 < CF_MAX_DMA) prefetch(kind_c, step / 3);
                 if constexpr (NT == 2)
                 {
                     if (more) ld_w(nxt, 0, step + AHEAD);
@@ -330,21 +354,26 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 }
             }
         };
-        auto contract_nt = [&](auto nt_c) __attribute__((always_inline))
+        if (tw < ntiles)
         {
-            if (prefetch_kind == 1) contract(nt_c, std::integral_constant<int, 1>());
-            else if (prefetch_kind == 2)
-                contract(nt_c, std::integral_constant<int, 2>());
+            if (two) contract(std::integral_constant<int, 2>());
             else
-                contract(nt_c, std::integral_constant<int, 0>());
-        };
-        if (two) contract_nt(std::integral_constant<int, 2>());
-        else
-            contract_nt(std::integral_constant<int, 1>());
+                contract(std::integral_constant<int, 1>());
+        }
 
-        // ---- epilogue: accumulator register v of lane l = channel n * 32 + 8 * (v / 4) + 4 * (l / 32) + v % 4 of pixel l % 32 --
-        const long long unit_base = ((long long) img * H + h0) * W * CF_K; // element offset of the unit's first output pixel
-        // one accumulator tile -> 16 consecutive channels of this lane's pixel, scaled
+        // the team is done with its tile: fetch the tile of its next unit (two units further down the run) underneath
+        // the epilogue and the other team's contraction
+        const int  img_done = img, h0_done = h0;
+        (void) img_done;
+        (void) h0_done;
+        advance();
+        if (row < row_end) advance();
+        cf_team_barrier(counter, 4 * ++barriers, lane);
+        if (row < row_end) issue_halo(img, h0, nrows);
+        if (tw >= ntiles) continue;
+
+        // ---- epilogue: accumulator register v of lane l = channel n * 32 + 8 * (v / 4) + 4 * (l / 32) + v % 4 of pixel
+        // l % 32; one v_permlane32_swap per register pair leaves the lane with channels n * 32 + kg * 16 + 0 .. 15 in order --
         auto gather = [&](int t, int n, float (&val)[16]) __attribute__((always_inline))
         {
 #pragma unroll
@@ -357,9 +386,6 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                     val[8 * g + i] = __uint_as_float(sw[0]);
                     val[8 * g + 4 + i] = __uint_as_float(sw[1]);
                 }
-        };
-        auto scale = [&](int n, float (&val)[16]) __attribute__((always_inline))
-        {
             if (has_alpha)
             {
 #pragma unroll
@@ -371,103 +397,57 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[n * 32 + kg * 16 + c]);
             }
         };
-        const bool scaled = has_alpha || col_exp != nullptr;
-        // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN (checked
-        // over all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x|
-        // over a lane's 16 values detects them and the unit is then converted again element by element.  Straight-line
-        // code on purpose: with one wavefront per SIMD only independent instructions hide each other's latency
-        auto store_bf16 = [&](auto relu_c, auto scale_c, auto nt_c) __attribute__((always_inline))
+#pragma unroll
+        for (int t = 0; t < 2; t++)
         {
-            constexpr bool RELU = decltype(relu_c)::value, SCALE = decltype(scale_c)::value;
-            constexpr int  NT = decltype(nt_c)::value;
-            float          val[NT][2][16];
-            uint32_t       pk[NT][2][8];
-            bool           special = false;
+            if (t == 1 && !two) break;
+            const int p = (tw + 4 * t) * 32 + (lane & 31);
 #pragma unroll
-            for (int t = 0; t < NT; t++)
-#pragma unroll
-                for (int n = 0; n < 2; n++)
+            for (int n = 0; n < 2; n++)
+            {
+                float val[16];
+                gather(t, n, val);
+                const long long idx = unit_base + (long long) p * CF_K + n * 32 + kg * 16;
+                if (bf16_fast)
                 {
-                    gather(t, n, val[t][n]);
-                    if (SCALE) scale(n, val[t][n]);
+                    // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN
+                    // (checked over all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are
+                    // rare: the sum of |x| over the lane's 16 values detects them and the block is then converted element
+                    // by element
                     float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int c = 0; c < 16; c++)
                     {
-                        if (RELU) val[t][n][c] = relu_ref(val[t][n][c]);
-                        sum[c & 3] += __builtin_fabsf(val[t][n][c]);
+                        if (cp.relu) val[c] = relu_ref(val[c]);
+                        sum[c & 3] += __builtin_fabsf(val[c]);
                     }
-                    special |= !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
-#pragma unroll
-                    for (int c = 0; c < 8; c++)
+                    const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
+                    uint32_t   pk[8];
+                    if (__builtin_amdgcn_ballot_w64(special) == 0)
                     {
-                        const cf_v2bf h = __builtin_convertvector(cf_v2f {val[t][n][2 * c], val[t][n][2 * c + 1]}, cf_v2bf);
-                        __builtin_memcpy(&pk[t][n][c], &h, 4);
-                    }
-                }
-            if (__builtin_amdgcn_ballot_w64(special) != 0)
-            {
-#pragma unroll
-                for (int t = 0; t < NT; t++)
-#pragma unroll
-                    for (int n = 0; n < 2; n++)
 #pragma unroll
                         for (int c = 0; c < 8; c++)
-                            pk[t][n][c] = fp32_to_bf16_rne(f2u(val[t][n][2 * c]), cp.clip_fp, cp.clip_inf_in) |
-                                          (fp32_to_bf16_rne(f2u(val[t][n][2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
-            }
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-            {
-                const int p = (wave + 4 * t) * 32 + (lane & 31);
-                if (p < npix)
-                {
-#pragma unroll
-                    for (int n = 0; n < 2; n++)
+                        {
+                            const cf_v2bf h = __builtin_convertvector(cf_v2f {val[2 * c], val[2 * c + 1]}, cf_v2bf);
+                            __builtin_memcpy(&pk[c], &h, 4);
+                        }
+                    }
+                    else
                     {
-                        cf_v4u* o = (cf_v4u*) ((uint16_t*) a.epi.out + unit_base + (long long) p * CF_K + n * 32 + kg * 16);
-                        o[0] = cf_v4u {pk[t][n][0], pk[t][n][1], pk[t][n][2], pk[t][n][3]};
-                        o[1] = cf_v4u {pk[t][n][4], pk[t][n][5], pk[t][n][6], pk[t][n][7]};
+#pragma unroll
+                        for (int c = 0; c < 8; c++)
+                            pk[c] = fp32_to_bf16_rne(f2u(val[2 * c]), cp.clip_fp, cp.clip_inf_in) |
+                                    (fp32_to_bf16_rne(f2u(val[2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
+                    }
+                    if (p < npix)
+                    {
+                        cf_v4u* o = (cf_v4u*) ((uint16_t*) a.epi.out + idx);
+                        o[0] = cf_v4u {pk[0], pk[1], pk[2], pk[3]};
+                        o[1] = cf_v4u {pk[4], pk[5], pk[6], pk[7]};
                     }
                 }
-            }
-        };
-        auto store_bf16_nt = [&](auto relu_c, auto scale_c) __attribute__((always_inline))
-        {
-            if (two) store_bf16(relu_c, scale_c, std::integral_constant<int, 2>());
-            else
-                store_bf16(relu_c, scale_c, std::integral_constant<int, 1>());
-        };
-        if (bf16_fast)
-        {
-            if (scaled)
-            {
-                if (cp.relu) store_bf16_nt(std::true_type(), std::true_type());
-                else
-                    store_bf16_nt(std::false_type(), std::true_type());
-            }
-            else
-            {
-                if (cp.relu) store_bf16_nt(std::true_type(), std::false_type());
-                else
-                    store_bf16_nt(std::false_type(), std::false_type());
-            }
-        }
-        else
-        {
-#pragma unroll
-            for (int t = 0; t < 2; t++)
-            {
-                if (t == 1 && !two) break;
-                const int p = (wave + 4 * t) * 32 + (lane & 31);
-#pragma unroll
-                for (int n = 0; n < 2; n++)
+                else if (p < npix)
                 {
-                    float val[16];
-                    gather(t, n, val);
-                    scale(n, val);
-                    if (p >= npix) continue;
-                    const long long idx = unit_base + (long long) p * CF_K + n * 32 + kg * 16;
                     if (!fused)
                     {
                         cf_v4f* o = (cf_v4f*) ((float*) a.epi.out + idx);
@@ -482,12 +462,9 @@ __global__ __launch_bounds__(256) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 }
             }
         }
-        row += nrows;
-        img = img1;
-        h0 = h1;
-        nrows = nrows1;
+        stores_in_flight = !fused ? (two ? 16 : 8) : bf16_fast ? (two ? 8 : 4) : 0;
+        (void) scaled;
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);
 }
 } // namespace
 
@@ -506,7 +483,7 @@ bool conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int 
 hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int W, const GemmEpilogue& epi, int num_cus, hipStream_t s)
 {
     static bool attr_done = false;
-    const int   lds_bytes = CF_WT_BYTES + 2 * (CF_TR + 2) * (W + 2) * 128;
+    const int   lds_bytes = CF_WT_BYTES + 2 * (CF_TR + 2) * (W + 2) * 128 + 16; // filter, one input tile per team, barrier counters
     if (!attr_done)
     {
         hipError_t e = hipFuncSetAttribute((const void*) conv_fwd_fast_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -523,7 +500,9 @@ hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int 
     const long long rows = (long long) B * H;
     if (rows > 0x7fffffffLL) return hipErrorInvalidValue;
     const int grid = (int) std::min<long long>((rows + CF_TR - 1) / CF_TR, num_cus > 0 ? num_cus : 256);
-    hipLaunchKernelGGL(conv_fwd_fast_kernel, dim3(grid), dim3(256), lds_bytes, s, a);
+    a.rows_per_wg = (int) (rows / grid);
+    a.rows_extra = (int) (rows % grid);
+    hipLaunchKernelGGL(conv_fwd_fast_kernel, dim3(grid), dim3(512), lds_bytes, s, a);
     return hipGetLastError();
 }
 
