@@ -4,11 +4,13 @@
 // Same arithmetic as the general kernel (gemm_impl.hpp): OCP fp8 MFMA with fp32 accumulation, Gaudi's exponent bias
 // folded into the epilogue multiplier.  What differs is the data movement, which is what bounds the general kernel:
 //
-//   tile        256 x 256 outputs per 256-lane workgroup; 4 wavefronts as 2 x 2, 128 x 128 each = 4 x 4 MFMA
-//               v_mfma_f32_32x32x64_f8f6f4 tiles -> 256 accumulator registers per lane (AGPRs), one wavefront per SIMD
+//   tile        256 x 256 outputs per 512-lane workgroup; 8 wavefronts as 2 x 4, 128 x 64 each = 4 x 2 MFMA
+//               v_mfma_f32_32x32x64_f8f6f4 tiles -> 128 accumulator registers per lane, two wavefronts per SIMD: a
+//               wavefront cannot issue anything while its own MFMA occupies it, so its neighbour's MFMAs are what
+//               cover its LDS reads, DMA requests and waits
 //   HBM/L2->LDS global_load_lds_dwordx4: 16 bytes per lane straight into LDS, no staging registers.  Ring of 4 stages of
 //               64 k-bytes (A 256 x 64 B + B 64 x 256 B = 32 KiB each, 128 KiB of LDS); stage t+3 is requested while
-//               stage t feeds the matrix cores, tracked with vmcnt (8 requests per lane and stage)
+//               stage t feeds the matrix cores, tracked with vmcnt (4 requests per lane and stage)
 //   LDS layout  16-byte chunks, placed so that every fragment read is bank-conflict free:
 //                 A (k contiguous): chunk (row r, c) at r*4 + (c ^ ((r>>2)&3))       -> ds_read_b128
 //                 B (n contiguous): chunk (k, cb)    at k*16 + ((cb + 2*(k&7)) & 15) -> ds_read_b64_tr_b8, the LDS
@@ -16,8 +18,11 @@
 //                   the 8 k-values of its own column, which is the operand layout of the MFMA (k packed per lane)
 //               the permutation is applied on the global-address side (each lane fetches the chunk that belongs at its
 //               LDS position), the DMA itself writes lanes in order
-//   schedule    one barrier per stage, placed right after an MFMA issue so that the 64 cycles of that MFMA cover it;
-//               fragment reads of stage t+1 and the 8 DMA requests of stage t+3 are interleaved one per MFMA
+//   schedule    one barrier per stage, placed right after an MFMA issue; every fragment register is refilled from
+//               stage t+1 right after its last use in stage t, the 4 DMA requests of stage t+3 ride along
+//   epilogue    the MFMA takes the B fragment as its first operand, so a lane's accumulator registers run along the
+//               output row: one v_permlane32_swap per register pair gives every lane 16 consecutive columns, written
+//               with 16-byte stores (bf16 through v_cvt_pk_bf16_f32 with an exact fall-back for NaN / inf / overflow)
 //   mapping     workgroup ids are dealt round-robin to the 8 XCDs; ids are remapped so that each XCD owns a compact
 //               8 x 4 block of tiles (12 operand panels through its L2 instead of 18)
 //
@@ -49,7 +54,7 @@ __device__ __forceinline__ void dma16(const void* g, uint32_t lds_off)
 
 struct Frags
 {
-    v8i a[4], b[4];
+    v8i a[4], b[2];
 };
 
 __device__ __forceinline__ void read_a(Frags& f, int i, const char* st, int wm, int lane)
@@ -62,7 +67,7 @@ __device__ __forceinline__ void read_a(Frags& f, int i, const char* st, int wm, 
 // B stored n-contiguous: transposed LDS reads
 __device__ __forceinline__ void read_b_tr(Frags& f, int j, const char* st, int wn, int lane)
 {
-    const int q = lane >> 4, cb = wn * 8 + j * 2 + (q & 1), g = q >> 1, rr = (lane & 15) >> 1, h = lane & 1;
+    const int q = lane >> 4, cb = wn * 4 + j * 2 + (q & 1), g = q >> 1, rr = (lane & 15) >> 1, h = lane & 1;
     v2i       t[4];
 #pragma unroll
     for (int tt = 0; tt < 4; tt++)
@@ -76,7 +81,7 @@ __device__ __forceinline__ void read_b_tr(Frags& f, int j, const char* st, int w
 // B stored k-contiguous (the "abt" form): same layout and reads as A
 __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int wn, int lane)
 {
-    const int r = wn * 128 + j * 32 + (lane & 31), c0 = 2 * (lane >> 5);
+    const int r = wn * 64 + j * 32 + (lane & 31), c0 = 2 * (lane >> 5);
     const v4i lo = *(const v4i*) (st + FBM * FBK + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + FBM * FBK + fa_pos(r, c0 + 1) * 16);
     f.b[j] = v8i {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
@@ -84,14 +89,14 @@ __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int w
 #define FENCE __builtin_amdgcn_sched_barrier(0)
 
 template<int FMT, bool B_KC>
-__global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_value)
+__global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_value)
 {
     (void) g_by_value;
     KARG GemmProblem& g = *(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr();
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     if (g.skip_flag && ((*g.skip_flag != 0u) == (g.skip_if != 0))) return;
 
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 1, wn = wave & 1;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
     const int tiles_n = g.N / FBN, tiles_m = g.M / FBM;
     int       tm, tn;
     {
@@ -121,22 +126,22 @@ __global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     const uint8_t*  B = (const uint8_t*) g.B.base + b_off;
     const uint32_t  lds_base = (uint32_t) (uintptr_t) lds;
 
-    v16f acc[4][4];
+    v16f acc[4][2];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     const int nk = g.K / FBK;
-    // per-lane global pointers of this wavefront's 4 + 4 request slots (they advance by one stage per step)
-    const uint8_t* ga[4];
-    const uint8_t* gb[4];
+    // per-lane global pointers of this wavefront's 2 + 2 request slots (they advance by one stage per step)
+    const uint8_t* ga[2];
+    const uint8_t* gb[2];
 #pragma unroll
-    for (int u = 0; u < 4; u++)
+    for (int u = 0; u < 2; u++)
     {
-        const int t = wave * 4 + u;
+        const int t = wave * 2 + u;
         {
             const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
             ga[u] = A + (size_t) (m0 + r) * lda + c * 16;
@@ -154,11 +159,11 @@ __global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     }
     auto issue_a = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
-        dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * FSTAGE + (wave * 4 + u) * 1024);
+        dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
     };
     auto issue_b = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
-        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * FBK * ldb), lds_base + slot * FSTAGE + FBM * FBK + (wave * 4 + u) * 1024);
+        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * FBK * ldb), lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
     };
     auto read_b = [&](Frags & f, int j, const char* st) __attribute__((always_inline))
     {
@@ -170,35 +175,34 @@ __global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     for (int t = 0; t < FNST - 1; t++)
     {
 #pragma unroll
-        for (int u = 0; u < 4; u++)
+        for (int u = 0; u < 2; u++)
         {
             issue_a(u, t, t);
             issue_b(u, t, t);
         }
     }
     // s_waitcnt immediate (gfx9): vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-    __builtin_amdgcn_s_waitcnt(0x4F70); // vmcnt(16): stage 0 has landed
+    __builtin_amdgcn_s_waitcnt(0x0F78); // vmcnt(8): stage 0 has landed
     __syncthreads();
-    Frags f0, f1;
+    Frags f;
 #pragma unroll
-    for (int i = 0; i < 4; i++)
-    {
-        read_a(f0, i, lds, wm, lane);
-        read_b(f0, i, lds);
-    }
+    for (int i = 0; i < 4; i++) read_a(f, i, lds, wm, lane);
+#pragma unroll
+    for (int j = 0; j < 2; j++) read_b(f, j, lds);
 
-#define MMA(i, j) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(cur.a[i], cur.b[j], acc[i][j], FMT & 1, (FMT >> 1) & 1, 0, 0, 0, 0)
+#define MMA(i, j) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0)
 #define RA(i) \
-    if (RN) read_a(nxt, i, st, wm, lane);
+    if (RN) read_a(f, i, st, wm, lane);
 #define RB(j) \
-    if (RN) read_b(nxt, j, st);
+    if (RN) read_b(f, j, st);
 #define LA(u) \
     if (LOADS) issue_a(u, t + FNST - 1, slot);
 #define LB(u) \
     if (LOADS) issue_b(u, t + FNST - 1, slot);
-    // One stage: 16 MFMAs on `cur`; after the first one wait until stage t+1 has landed in every wavefront's view
-    // (WAITC leaves the younger stages in flight) and fetch its fragments into `nxt`; request stage t+3.
-    auto step = [&](int t, Frags& cur, Frags& nxt, auto waitc, auto loads, auto readnext) __attribute__((always_inline))
+    // One stage: 8 MFMAs; after the first one wait until stage t+1 has landed in every wavefront's view (WAITC leaves the
+    // younger stage in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
+    // other wavefront on the SIMD covers the tail of that latency); request stage t+3.
+    auto step = [&](int t, auto waitc, auto loads, auto readnext) __attribute__((always_inline))
     {
         constexpr int  WAITC = decltype(waitc)::value;
         constexpr bool LOADS = decltype(loads)::value;
@@ -213,38 +217,30 @@ __global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_val
             __builtin_amdgcn_s_barrier();
         }
         FENCE;
-        MMA(0, 1); RA(0) LA(0) FENCE;
-        MMA(0, 2); RA(1) FENCE;
-        MMA(0, 3); RA(2) LA(1) FENCE;
-        MMA(1, 0); RA(3) FENCE;
-        MMA(1, 1); RB(0) LA(2) FENCE;
-        MMA(1, 2); FENCE;
-        MMA(1, 3); RB(1) LA(3) FENCE;
-        MMA(2, 0); FENCE;
-        MMA(2, 1); RB(2) LB(0) FENCE;
-        MMA(2, 2); FENCE;
-        MMA(2, 3); RB(3) LB(1) FENCE;
-        MMA(3, 0); FENCE;
-        MMA(3, 1); LB(2) FENCE;
-        MMA(3, 2); FENCE;
-        MMA(3, 3); LB(3) FENCE;
-        if (RN) __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): `nxt` is complete, this wavefront is done with the stage
+        MMA(0, 1); FENCE;
+        RA(0) LA(0) MMA(1, 0); FENCE;
+        MMA(1, 1); FENCE;
+        RA(1) LA(1) MMA(2, 0); FENCE;
+        MMA(2, 1); FENCE;
+        RA(2) LB(0) MMA(3, 0); FENCE;
+        RB(0) LB(1) MMA(3, 1); FENCE;
+        RA(3) RB(1) FENCE;
     };
-    using W8 = std::integral_constant<int, 0x0F78>; // vmcnt(8)
+    using W8 = std::integral_constant<int, 0x0F74>; // vmcnt(4): one stage of this wavefront's requests may still be in flight
     using W0 = std::integral_constant<int, 0x0F70>; // vmcnt(0)
     using T = std::true_type;
     using F = std::false_type;
     int t = 0;
     for (; t + 5 <= nk; t += 2)
     {
-        step(t, f0, f1, W8 {}, T {}, T {});
-        step(t + 1, f1, f0, W8 {}, T {}, T {});
+        step(t, W8 {}, T {}, T {});
+        step(t + 1, W8 {}, T {}, T {});
     }
     // t == nk - 4 (nk is even and >= 6)
-    step(t, f0, f1, W8 {}, T {}, T {});     // requests the last stage
-    step(t + 1, f1, f0, W8 {}, F {}, T {}); // stage nk-2 needed, stage nk-1 may be in flight
-    step(t + 2, f0, f1, W0 {}, F {}, T {});
-    step(t + 3, f1, f0, W0 {}, F {}, F {});
+    step(t, W8 {}, T {}, T {});     // requests the last stage
+    step(t + 1, W8 {}, F {}, T {}); // stage nk-2 needed, stage nk-1 may be in flight
+    step(t + 2, W0 {}, F {}, T {});
+    step(t + 3, W0 {}, F {}, F {});
 #undef MMA
 #undef RA
 #undef RB
@@ -252,8 +248,10 @@ __global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_val
 #undef LB
 
     // ---- epilogue: alpha, per-column power of two, relu, cast, store (same conversion functions as the general kernel).
-    // The output-type dispatch sits outside the fully unrolled accumulator walk so that the accumulators stay in
-    // registers.  Addresses are a uniform 64-bit tile base plus 32-bit lane offsets (one add per element).
+    // The matrix-core operands are swapped (B fragment first), so accumulator register v of lane l is output column
+    // 8 * (v / 4) + 4 * (l / 32) + v % 4 of row l % 32 of its 32 x 32 block: one v_permlane32_swap per register pair leaves
+    // every lane with 16 consecutive columns of one row, stored 16 bytes at a time.  The output-type dispatch sits
+    // outside the unrolled block walk so that the accumulators stay in registers.
     const long long c_off = b0 * g.epi.batch_stride[0] + b1 * g.epi.batch_stride[1] + b2 * g.epi.batch_stride[2];
     const long long ldc = g.epi.ld;
     const bool      has_alpha = g.epi.has_alpha != 0;
@@ -262,109 +260,151 @@ __global__ __launch_bounds__(256) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     const bool      relu = g.epi.fused && g.epi.cast.relu;
     const int       dt = g.epi.fused ? g.epi.out_dtype : DT_FP32;
     const int       esz = (dt == DT_FP32) ? 4 : (dt == DT_BF16 ? 2 : 1);
-    char*           tile_base = (char*) g.epi.out + (c_off + (long long) m0 * ldc + n0) * esz; // uniform
-    const uint32_t  ldcb = (uint32_t) ldc * esz;                                              // bytes per output row
     const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
                            g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
-    // value of accumulator (i, j, v) after the power-of-two factors and relu
-    auto value = [&](int i, int j, int v, float cs) __attribute__((always_inline))
+    const int       kg = lane >> 5;
+    // element offset of this lane's first value in block (0, 0): row m0 + wm * 128 + lane % 32, column n0 + wn * 64 + 16 kg
+    const long long lane_elem = c_off + (long long) (m0 + wm * 128 + (lane & 31)) * ldc + n0 + wn * 64 + kg * 16;
+    // block (i, j) -> the lane's 16 values after the power-of-two factors and relu
+    auto gather = [&](int i, int j, float (&val)[16]) __attribute__((always_inline))
     {
-        float x = acc[i][j][v];
-        if (has_alpha) x *= alpha;
-        if (col_exp) x *= cs;
-        if (relu) x = relu_ref(x);
-        return x;
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+            {
+                const float lo = acc[i][j][4 * q + r], hi = acc[i][j][8 + 4 * q + r];
+                const auto  sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                val[8 * q + r] = __uint_as_float(sw[0]);
+                val[8 * q + 4 + r] = __uint_as_float(sw[1]);
+            }
+        if (has_alpha)
+        {
+#pragma unroll
+            for (int c = 0; c < 16; c++) val[c] *= alpha;
+        }
+        if (col_exp)
+        {
+#pragma unroll
+            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
+        }
+        if (relu)
+        {
+#pragma unroll
+            for (int c = 0; c < 16; c++) val[c] = relu_ref(val[c]);
+        }
     };
-    // generic walk: one store per element
     auto walk = [&](auto store) __attribute__((always_inline))
     {
-        const uint32_t lane_off = (uint32_t) (wm * 128 + 4 * (lane >> 5)) * ldcb + (uint32_t) (wn * 128 + (lane & 31)) * esz;
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-        {
-            float cs = 1.0f;
-            if (col_exp) cs = pow2_of(col_exp[n0 + wn * 128 + j * 32 + (lane & 31)]);
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int v = 0; v < 16; v++)
-                    store(tile_base + (lane_off + (uint32_t) (i * 32 + 8 * (v >> 2) + (v & 3)) * ldcb + (uint32_t) (j * 32 * esz)), value(i, j, v, cs));
-        }
-    };
-    if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
-        walk([&](char* p, float x) __attribute__((always_inline)) { *(float*) p = x; });
-    else if (dt == DT_BF16 && g.epi.fast_cast)
-    {
-        // bf16, round to nearest even.  Lanes l and l^1 hold neighbouring columns: they swap one packed pair of rows
-        // through DPP so that every lane stores whole dwords (two columns of one row).  NaN, inf and values that round
-        // to inf are rare: a per-tile maximum of |x| detects them and that tile takes the element-wise conversion.
-        const uint32_t odd = lane & 1;
-        const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
-        const uint32_t lane_off = (uint32_t) (wm * 128 + 4 * (lane >> 5) + odd) * ldcb + (uint32_t) (wn * 128 + (lane & 30)) * 2;
-        const uint32_t lane_off1 = (uint32_t) (wm * 128 + 4 * (lane >> 5)) * ldcb + (uint32_t) (wn * 128 + (lane & 31)) * 2;
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-        {
-            float cs = 1.0f;
-            if (col_exp) cs = pow2_of(col_exp[n0 + wn * 128 + j * 32 + (lane & 31)]);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int j = 0; j < 2; j++)
             {
-                uint32_t sum[16], mx = 0;
+                float val[16];
+                gather(i, j, val);
+                store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
+            }
+    };
+    typedef float    e_v4f __attribute__((ext_vector_type(4)));
+    typedef uint32_t e_v4u __attribute__((ext_vector_type(4)));
+    typedef float    e_v2f __attribute__((ext_vector_type(2)));
+    typedef __bf16   e_v2bf __attribute__((ext_vector_type(2)));
+    if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
+        walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
+            e_v4f* o = (e_v4f*) ((float*) g.epi.out + idx);
 #pragma unroll
-                for (int v = 0; v < 16; v++)
-                {
-                    const uint32_t u = f2u(value(i, j, v, cs));
-                    mx = max(mx, u & 0x7FFFFFFFu);
-                    sum[v] = u + 0x7FFFu + ((u >> 16) & 1u); // bf16 code in the high half
-                }
-                if (__builtin_amdgcn_ballot_w64(mx >= 0x7F7F8000u) == 0)
-                {
+            for (int c = 0; c < 4; c++) o[c] = e_v4f {val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3]};
+        });
+    else if (dt == DT_BF16 && g.epi.fast_cast)
+        // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN (checked over
+        // all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x| over
+        // the lane's 16 values detects them and the block is then converted element by element
+        walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
+            float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                    for (int v = 0; v < 16; v += 2)
-                    {
-                        const uint32_t mine = __builtin_amdgcn_perm(sum[v + 1], sum[v], 0x07060302u); // rows v, v+1 of my column
-                        const uint32_t theirs = (uint32_t) __builtin_amdgcn_update_dpp(0, (int) mine, 0xB1, 0xF, 0xF, false); // lane ^ 1
-                        // even lane: row v = (my col, next col); odd lane: row v+1 = (previous col, my col)
-                        const uint32_t word = __builtin_amdgcn_perm(theirs, mine, sel);
-                        *(uint32_t*) (tile_base + (lane_off + (uint32_t) (i * 32 + 8 * (v >> 2) + (v & 3)) * ldcb + (uint32_t) (j * 64))) = word;
-                    }
-                }
-                else
-                {
+            for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
+            const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
+            uint32_t   pk[8];
+            if (__builtin_amdgcn_ballot_w64(special) == 0)
+            {
 #pragma unroll
-                    for (int v = 0; v < 16; v++)
-                        *(uint16_t*) (tile_base + (lane_off1 + (uint32_t) (i * 32 + 8 * (v >> 2) + (v & 3)) * ldcb + (uint32_t) (j * 64))) =
-                            (uint16_t) fp32_to_bf16_rne(f2u(value(i, j, v, cs)), cp.clip_fp, cp.clip_inf_in);
+                for (int c = 0; c < 8; c++)
+                {
+                    const e_v2bf h = __builtin_convertvector(e_v2f {val[2 * c], val[2 * c + 1]}, e_v2bf);
+                    __builtin_memcpy(&pk[c], &h, 4);
                 }
             }
-        }
+            else
+            {
+#pragma unroll
+                for (int c = 0; c < 8; c++)
+                    pk[c] = fp32_to_bf16_rne(f2u(val[2 * c]), cp.clip_fp, cp.clip_inf_in) | (fp32_to_bf16_rne(f2u(val[2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
+            }
+            e_v4u* o = (e_v4u*) ((uint16_t*) g.epi.out + idx);
+            o[0] = e_v4u {pk[0], pk[1], pk[2], pk[3]};
+            o[1] = e_v4u {pk[4], pk[5], pk[6], pk[7]};
+        });
+    else if ((dt == DT_FP8_143 || dt == DT_FP8_152) && g.epi.fast_cast)
+    {
+        auto fp8_store = [&](auto m_c) __attribute__((always_inline))
+        {
+            constexpr int MAN = decltype(m_c)::value;
+            walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
+                uint32_t pk[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                {
+                    pk[c] = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) pk[c] |= (fp32_to_fp8_rne_mode0<MAN>(f2u(val[4 * c + e]), cp.exp_bias, cp.clip_fp, cp.clip_inf_in) & 0xFFu) << (8 * e);
+                }
+                *(e_v4u*) ((uint8_t*) g.epi.out + idx) = e_v4u {pk[0], pk[1], pk[2], pk[3]};
+            });
+        };
+        if (dt == DT_FP8_143) fp8_store(std::integral_constant<int, 3>());
+        else
+            fp8_store(std::integral_constant<int, 2>());
     }
-    else if (dt == DT_FP8_143 && g.epi.fast_cast)
-        walk([&](char* p, float x) __attribute__((always_inline)) { *(uint8_t*) p = (uint8_t) fp32_to_fp8_rne_mode0<3>(f2u(x), cp.exp_bias, cp.clip_fp, cp.clip_inf_in); });
-    else if (dt == DT_FP8_152 && g.epi.fast_cast)
-        walk([&](char* p, float x) __attribute__((always_inline)) { *(uint8_t*) p = (uint8_t) fp32_to_fp8_rne_mode0<2>(f2u(x), cp.exp_bias, cp.clip_fp, cp.clip_inf_in); });
     else
     {
-        // rare cast settings: element-wise through the out-of-line generic converter (relu is applied there)
-        const uint32_t lane_row = wm * 128 + 4 * (lane >> 5), lane_col = wn * 128 + (lane & 31);
+        // rare cast settings: element-wise through the out-of-line generic converter (which applies relu itself)
+#pragma unroll 1
+        for (int i = 0; i < 4; i++)
+#pragma unroll 1
+            for (int j = 0; j < 2; j++)
+            {
+                float val[16];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-        {
-            float cs = 1.0f;
-            if (col_exp) cs = pow2_of(col_exp[n0 + lane_col + j * 32]);
+                for (int q = 0; q < 2; q++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+                    for (int r = 0; r < 4; r++)
+                    {
+                        // (dynamic block index: read the accumulators through a switch-free copy)
+                        float lo = 0.0f, hi = 0.0f;
 #pragma unroll
-                for (int v = 0; v < 16; v++)
+                        for (int ii = 0; ii < 4; ii++)
+#pragma unroll
+                            for (int jj = 0; jj < 2; jj++)
+                                if (ii == i && jj == j)
+                                {
+                                    lo = acc[ii][jj][4 * q + r];
+                                    hi = acc[ii][jj][8 + 4 * q + r];
+                                }
+                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                        val[8 * q + r] = __uint_as_float(sw[0]);
+                        val[8 * q + 4 + r] = __uint_as_float(sw[1]);
+                    }
+                for (int c = 0; c < 16; c++)
                 {
-                    float x = acc[i][j][v];
+                    float x = val[c];
                     if (has_alpha) x *= alpha;
-                    if (col_exp) x *= cs;
-                    store_out_slow(g.epi, c_off + (long long) (m0 + lane_row + i * 32 + 8 * (v >> 2) + (v & 3)) * ldc + n0 + lane_col + j * 32, x);
+                    if (col_exp) x *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
+                    store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
                 }
-        }
+            }
     }
+    (void) esz;
 }
 
 template<int FMT>
@@ -379,9 +419,9 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
         if (e != hipSuccess) return e;
         attr_done[bkc] = true;
     }
-    if (bkc) hipLaunchKernelGGL((gemm_fp8_fast_kernel<FMT, true>), grid, dim3(256), FNST * FSTAGE, s, p);
+    if (bkc) hipLaunchKernelGGL((gemm_fp8_fast_kernel<FMT, true>), grid, dim3(512), FNST * FSTAGE, s, p);
     else
-        hipLaunchKernelGGL((gemm_fp8_fast_kernel<FMT, false>), grid, dim3(256), FNST * FSTAGE, s, p);
+        hipLaunchKernelGGL((gemm_fp8_fast_kernel<FMT, false>), grid, dim3(512), FNST * FSTAGE, s, p);
     return hipGetLastError();
 }
 } // namespace
@@ -393,13 +433,14 @@ bool gemm_fp8_fast_applicable(const GemmProblem& p)
     if (!p.A.k_contig || !p.A.vec_ok || !p.B.vec_ok) return false;
     if (p.split_k > 1) return false;
     if (p.M % FBM || p.N % FBN || p.K % (2 * FBK) || p.K < 6 * FBK) return false;
-    // epilogue: 32-bit byte offsets inside a tile, dword stores of bf16 pairs
-    if (p.epi.ld <= 0 || p.epi.ld * 4 * FBM >= (1ll << 31)) return false;
-    if (p.epi.fused && p.epi.out_dtype == DT_BF16)
+    // epilogue: 16-byte stores of 16 consecutive output columns (4 for fp32)
+    if (p.epi.ld <= 0) return false;
     {
-        if ((p.epi.ld & 1) || ((uintptr_t) p.epi.out & 3)) return false;
+        const int out_dt = p.epi.fused ? p.epi.out_dtype : DT_FP32;
+        const int per16 = out_dt == DT_FP32 ? 4 : (out_dt == DT_BF16 ? 8 : 16); // elements per 16 bytes
+        if ((p.epi.ld % per16) || ((uintptr_t) p.epi.out & 15)) return false;
         for (int d = 0; d < 3; d++)
-            if (p.epi.batch_stride[d] & 1) return false;
+            if (p.epi.batch_stride[d] % per16) return false;
     }
     return true;
 }
