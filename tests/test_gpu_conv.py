@@ -123,3 +123,38 @@ def test_conv_fwd_fast_path_vs_oracle(calc, orc, B, H, W):
     want16 = np.zeros(want.size, np.uint16)
     assert orc.orc_cast_from_fp32(want16.ctypes.data, abi.BF16, 0, 0, got.ctypes.data, got.size, 1, None, 0, 1, 0, 1, 0, 0) == 0
     assert np.array_equal(out.cpu().numpy().view(np.uint16), want16)
+
+
+@pytest.mark.parametrize("relu,clip", [(False, False), (True, False), (False, True), (True, True)])
+def test_conv_fwd_fast_path_special_values(calc, orc, relu, clip):
+    """inf, NaN and huge activations through the specialised forward kernel with an unscaled bf16 epilogue: the
+    blocks that hold NaN / inf / overflow leave the hardware-convert path for the exact converter; bit-exact against the
+    oracle cast (relu, clipping) of the kernel's own fp32 accumulators."""
+    import torch
+    from intel_gaudi3_software_amd import Epilogue
+    from helpers import to_bf16_bits
+    rng = np.random.default_rng(900)
+    B, H, W = 2, 9, 21
+    xs, ws, ys = [64, W, H, 1, B], [64, 64, 3, 3, 1], [64, W, H, 1, B]
+    x = to_bf16_bits(rng.standard_normal(int(np.prod(xs))))
+    w = to_bf16_bits(rng.standard_normal(int(np.prod(ws))) * 0.05)
+    xv = x.reshape(B, H, W, 64)
+    xv[0, 2, 3, 5] = 0x7F80   # +inf
+    xv[0, 6, 17, 9] = 0xFF80  # -inf
+    xv[1, 4, 4, 0] = 0x7FC0   # NaN
+    xv[1, 7, 12, :] = 0x7F00  # 1.7e38 in every channel: sums overflow bf16 and fp32
+    tx, tw = torch.from_numpy(x.view(np.int16)).cuda(), torch.from_numpy(w.view(np.int16)).cuda()
+    n = int(np.prod(ys))
+    acc = torch.zeros(n, dtype=torch.float32, device="cuda")
+    out = torch.zeros(n, dtype=torch.int16, device="cuda")
+    X, Wt = MmeSimTensor(xs, 5, abi.BF16, tx), MmeSimTensor(ws, 5, abi.BF16, tw)
+    cp = ConvolutionParams(2, [1, 1, 0, 0], [1, 1, 1, 1], [1, 1, 1, 1])
+    calc.doConvolution(MmeSimTensor(ys, 5, abi.FP32, acc), X, Wt, MmeSimTensor(ys, 5, abi.FP32, acc), cp, abi.OP_FWD)
+    calc.doConvolution(MmeSimTensor(ys, 5, abi.BF16, out), X, Wt, MmeSimTensor(ys, 5, abi.BF16, out), cp, abi.OP_FWD,
+                       epilogue=Epilogue(relu=relu, clipFp=clip))
+    calc.synchronize()
+    got = acc.cpu().numpy()
+    assert np.isnan(got).any() and np.isinf(got).any()
+    want16 = np.zeros(n, np.uint16)
+    assert orc.orc_cast_from_fp32(want16.ctypes.data, abi.BF16, 0, 0, got.ctypes.data, n, 0, None, 0, int(relu), 0, int(clip), 0, 0) == 0
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want16)

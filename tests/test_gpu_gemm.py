@@ -250,3 +250,32 @@ def test_fp8_fast_kernel_fused_epilogue_bit_exact(calc, orc):
                                       1, 0, 0) == 0
         got = out.cpu().numpy()
         assert np.array_equal(got.view(want.dtype), want)
+
+
+@pytest.mark.parametrize("clip", [False, True])
+def test_fp8_fast_kernel_epilogue_overflow_takes_exact_conversion(calc, orc, clip):
+    """A descale that pushes part of the accumulators beyond the bf16 range: those blocks leave the hardware-convert path
+    for the exact converter (inf without clipping, the largest normal with it); bit-exact against the oracle cast."""
+    import torch
+    rng = np.random.default_rng(67)
+    M, N, K = 256, 256, 384
+    a = random_operand(rng, abi.FP8_143, M * K, orc, 7)
+    b = random_operand(rng, abi.FP8_143, N * K, orc, 7)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    X, W = MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7), MmeSimTensor([N, K], 2, abi.FP8_143, tb, 7)
+    acc = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, acc), X, W, abi.OP_AB)
+    # per-column exponents: most columns stay finite, some overflow to inf in fp32, some only in bf16
+    col = np.zeros(N, np.int32)
+    col[::7] = 126
+    col[3::11] = 124
+    out = torch.zeros(M * N, dtype=torch.int16, device="cuda")
+    epi = Epilogue(scale_exp=0, col_scale_exp=torch.from_numpy(col).cuda(), clipFp=clip)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.BF16, out), X, W, abi.OP_AB, epilogue=epi)
+    calc.synchronize()
+    acc_h = acc.cpu().numpy()
+    want = np.zeros(M * N, np.uint16)
+    assert orc.orc_cast_from_fp32(want.ctypes.data, abi.BF16, 0, 0, acc_h.ctypes.data, M * N, 0, col.ctypes.data, N, 0, 0, int(clip), 0, 0) == 0
+    got = out.cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+    assert (np.any((want & 0x7FFF) == 0x7F7F) if clip else np.any((want & 0x7FFF) == 0x7F80))
