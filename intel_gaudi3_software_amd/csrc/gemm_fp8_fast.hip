@@ -1,8 +1,9 @@
-// gemm_fp8_fast.hip -- the fp8 contraction for large aligned problems (the headline path: fp8_143 / fp8_152 operands,
-// M and N multiples of 256, K a multiple of 128 and >= 384, 16-byte aligned rows).
+// gemm_fp8_fast.hip -- the contraction for large aligned problems (the headline path: fp8_143 / fp8_152 operands, and
+// bf16 through the same code; M and N multiples of 256, K a multiple of 128 bytes and >= 384 bytes, 16-byte aligned rows).
 //
-// Same arithmetic as the general kernel (gemm_impl.hpp): OCP fp8 MFMA with fp32 accumulation, Gaudi's exponent bias
-// folded into the epilogue multiplier.  What differs is the data movement, which is what bounds the general kernel:
+// Same arithmetic as the general kernel (gemm_impl.hpp): OCP fp8 (or bf16) MFMA with fp32 accumulation, Gaudi's exponent
+// bias folded into the epilogue multiplier.  bf16 differs only in the matrix-core instruction (two v_mfma_f32_32x32x16_bf16
+// per 64-byte stage and tile pair) and in the transposing read of an n-contiguous B (ds_read_b64_tr_b16).  What differs is the data movement, which is what bounds the general kernel:
 //
 //   tile        256 x 256 outputs per 512-lane workgroup; 8 wavefronts as 2 x 4, 128 x 64 each = 4 x 2 MFMA
 //               v_mfma_f32_32x32x64_f8f6f4 tiles -> 128 accumulator registers per lane, two wavefronts per SIMD: a
@@ -78,6 +79,29 @@ __device__ __forceinline__ void read_b_tr(Frags& f, int j, const char* st, int w
     f.b[j] = v8i {t[0].x, t[0].y, t[1].x, t[1].y, t[2].x, t[2].y, t[3].x, t[3].y};
 }
 
+// bf16, B stored n-contiguous: a stage is 32 k-rows x 256 columns x 2 B = 32 chunks of 16 B per row, the 32-byte blocks of a
+// row XOR-swizzled by k & 3.  ds_read_b64_tr_b16: within a group of 16 lanes, lane q addresses the 8-byte piece q % 4 of
+// row q / 4 and receives 4 consecutive k of its own column.  The fragment's k order ({0-7, 16-23} then {8-15, 24-31}
+// for the two lane halves) is the one the k-contiguous reads of the other operand produce.
+__device__ __forceinline__ void read_b_tr16(Frags& f, int j, const char* st, int wn, int lane)
+{
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wn * 4 + j * 2 + (g & 1);
+    union
+    {
+        v4s h4[4];
+        v8i v;
+    } u;
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+    {
+        // reads 0, 1 -> k = 16 h + 0 .. 7 (first MFMA), reads 2, 3 -> k = 16 h + 8 .. 15 (second MFMA)
+        const int k = 16 * h + 4 * tt + (q >> 2);
+        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + FBM * FBK + k * 512 + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
+    }
+    f.b[j] = u.v;
+}
+
 // B stored k-contiguous (the "abt" form): same layout and reads as A
 __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int wn, int lane)
 {
@@ -88,11 +112,11 @@ __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int w
 
 #define FENCE __builtin_amdgcn_sched_barrier(0)
 
-template<int FMT, bool B_KC>
-__global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_value)
+// ES = 1: fp8 (FMT selects e4m3 / e5m2 per operand), ES = 2: bf16.  Everything up to the matrix-core instruction is
+// byte-based and shared: a stage is 64 bytes of k per row for both.
+template<int ES, int FMT, bool B_KC>
+__device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
-    (void) g_by_value;
-    KARG GemmProblem& g = *(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr();
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     if (g.skip_flag && ((*g.skip_flag != 0u) == (g.skip_if != 0))) return;
 
@@ -120,10 +144,10 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     const long long a_off = b0 * g.A.batch_stride[0] + b1 * g.A.batch_stride[1] + b2 * g.A.batch_stride[2];
     const long long b_off = b0 * g.B.batch_stride[0] + b1 * g.B.batch_stride[1] + b2 * g.B.batch_stride[2];
     const int       m0 = tm * FBM, n0 = tn * FBN;
-    const long long lda = g.A.stride_f;
-    const long long ldb = B_KC ? g.B.stride_f : g.B.stride_k;
-    const uint8_t*  A = (const uint8_t*) g.A.base + a_off;
-    const uint8_t*  B = (const uint8_t*) g.B.base + b_off;
+    const long long lda = g.A.stride_f * ES; // bytes
+    const long long ldb = (B_KC ? g.B.stride_f : g.B.stride_k) * ES;
+    const uint8_t*  A = (const uint8_t*) g.A.base + a_off * ES;
+    const uint8_t*  B = (const uint8_t*) g.B.base + b_off * ES;
     const uint32_t  lds_base = (uint32_t) (uintptr_t) lds;
 
     v16f acc[4][2];
@@ -134,7 +158,8 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    const int nk = g.K / FBK;
+    // split-k: blockIdx.z takes an equal slice of the stages and writes raw partial sums to the workspace
+    const int nk = g.K * ES / FBK / (g.split_k > 1 ? g.split_k : 1), kt_begin = (g.split_k > 1 ? (int) blockIdx.z : 0) * nk;
     // per-lane global pointers of this wavefront's 2 + 2 request slots (they advance by one stage per step)
     const uint8_t* ga[2];
     const uint8_t* gb[2];
@@ -144,17 +169,22 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
         const int t = wave * 2 + u;
         {
             const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-            ga[u] = A + (size_t) (m0 + r) * lda + c * 16;
+            ga[u] = A + (size_t) (m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
         }
         if (B_KC)
         {
             const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-            gb[u] = B + (size_t) (n0 + r) * ldb + c * 16;
+            gb[u] = B + (size_t) (n0 + r) * ldb + c * 16 + (size_t) kt_begin * FBK;
+        }
+        else if (ES == 1)
+        {
+            const int k = t * 4 + (lane >> 4), p = lane & 15, cb = (p - 2 * (k & 7)) & 15;
+            gb[u] = B + (size_t) (k + kt_begin * FBK) * ldb + n0 + cb * 16;
         }
         else
         {
-            const int k = t * 4 + (lane >> 4), p = lane & 15, cb = (p - 2 * (k & 7)) & 15;
-            gb[u] = B + (size_t) k * ldb + n0 + cb * 16;
+            const int k = t * 2 + (lane >> 5), p = lane & 31, chunk = p ^ ((k & 3) << 1);
+            gb[u] = B + (size_t) (k + kt_begin * (FBK / 2)) * ldb + n0 * 2 + chunk * 16;
         }
     }
     auto issue_a = [&](int u, int stage, int slot) __attribute__((always_inline))
@@ -163,13 +193,15 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     };
     auto issue_b = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
-        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * FBK * ldb), lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
+        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
     };
     auto read_b = [&](Frags & f, int j, const char* st) __attribute__((always_inline))
     {
         if (B_KC) read_b_kc(f, j, st, wn, lane);
-        else
+        else if (ES == 1)
             read_b_tr(f, j, st, wn, lane);
+        else
+            read_b_tr16(f, j, st, wn, lane);
     };
 
     for (int t = 0; t < FNST - 1; t++)
@@ -190,7 +222,24 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
 #pragma unroll
     for (int j = 0; j < 2; j++) read_b(f, j, lds);
 
-#define MMA(i, j) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0)
+    auto mma = [&](int i, int j) __attribute__((always_inline))
+    {
+        if constexpr (ES == 1)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
+        else
+        {
+            union
+            {
+                v8i  v;
+                v8bf h[2];
+            } ua, ub;
+            ua.v = f.a[i];
+            ub.v = f.b[j];
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ub.h[0], ua.h[0], acc[i][j], 0, 0, 0);
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ub.h[1], ua.h[1], acc[i][j], 0, 0, 0);
+        }
+    };
+#define MMA(i, j) mma(i, j)
 #define RA(i) \
     if (RN) read_a(f, i, st, wm, lane);
 #define RB(j) \
@@ -310,7 +359,35 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     typedef uint32_t e_v4u __attribute__((ext_vector_type(4)));
     typedef float    e_v2f __attribute__((ext_vector_type(2)));
     typedef __bf16   e_v2bf __attribute__((ext_vector_type(2)));
-    if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
+    if (g.split_k > 1)
+    {
+        // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
+        float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N +
+                    (long long) (m0 + wm * 128 + (lane & 31)) * g.N + n0 + wn * 64 + kg * 16;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+            {
+                e_v4f* o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
+#pragma unroll
+                for (int q = 0; q < 2; q++)
+                {
+                    float lo4[4], hi4[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                    {
+                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint((float) acc[i][j][4 * q + r]),
+                                                                         __float_as_uint((float) acc[i][j][8 + 4 * q + r]), false, false);
+                        lo4[r] = __uint_as_float(sw[0]);
+                        hi4[r] = __uint_as_float(sw[1]);
+                    }
+                    o[2 * q] = e_v4f {lo4[0], lo4[1], lo4[2], lo4[3]};
+                    o[2 * q + 1] = e_v4f {hi4[0], hi4[1], hi4[2], hi4[3]};
+                }
+            }
+    }
+    else if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
         walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
             e_v4f* o = (e_v4f*) ((float*) g.epi.out + idx);
 #pragma unroll
@@ -407,6 +484,37 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     (void) esz;
 }
 
+template<int FMT, bool B_KC>
+__global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_value)
+{
+    (void) g_by_value;
+    gemm_fast_body<1, FMT, B_KC>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+}
+
+template<bool B_KC>
+__global__ __launch_bounds__(512) void gemm_bf16_fast_kernel(GemmProblem g_by_value)
+{
+    (void) g_by_value;
+    gemm_fast_body<2, 0, B_KC>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+}
+
+hipError_t launch_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
+{
+    static bool attr_done[2] = {false, false};
+    const bool  bkc = p.B.k_contig != 0;
+    const void* fn = bkc ? (const void*) gemm_bf16_fast_kernel<true> : (const void*) gemm_bf16_fast_kernel<false>;
+    if (!attr_done[bkc])
+    {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, FNST * FSTAGE);
+        if (e != hipSuccess) return e;
+        attr_done[bkc] = true;
+    }
+    if (bkc) hipLaunchKernelGGL((gemm_bf16_fast_kernel<true>), grid, dim3(512), FNST * FSTAGE, s, p);
+    else
+        hipLaunchKernelGGL((gemm_bf16_fast_kernel<false>), grid, dim3(512), FNST * FSTAGE, s, p);
+    return hipGetLastError();
+}
+
 template<int FMT>
 hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 {
@@ -428,11 +536,17 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 
 bool gemm_fp8_fast_applicable(const GemmProblem& p)
 {
-    if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152)) return false;
+    if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152 || p.dtype == DT_BF16)) return false;
+    const int es = p.dtype == DT_BF16 ? 2 : 1;
     if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN) return false;
     if (!p.A.k_contig || !p.A.vec_ok || !p.B.vec_ok) return false;
-    if (p.split_k > 1) return false;
-    if (p.M % FBM || p.N % FBN || p.K % (2 * FBK) || p.K < 6 * FBK) return false;
+    if (p.M % FBM || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
+    if (p.split_k > 1)
+    {
+        // every slice an even number of stages, at least 6
+        const int nk = p.K * es / FBK;
+        if (nk % (2 * p.split_k) || nk / p.split_k < 6) return false;
+    }
     // epilogue: 16-byte stores of 16 consecutive output columns (4 for fp32)
     if (p.epi.ld <= 0) return false;
     {
@@ -445,10 +559,26 @@ bool gemm_fp8_fast_applicable(const GemmProblem& p)
     return true;
 }
 
+int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
+{
+    GemmProblem q = p;
+    q.split_k = 1;
+    if (!gemm_fp8_fast_applicable(q)) return 0;
+    const long long tiles = (long long) (p.M / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
+    const int       nk = p.K * (p.dtype == DT_BF16 ? 2 : 1) / FBK;
+    int             best = 1;
+    // Splitting pays only while the tiles leave most of the chip idle: each slice costs a pass of the fp32 output through
+    // the workspace and the reduction kernel.  Every slice keeps an even number of stages, at least 6.
+    for (int s = 2; s <= 4 && tiles * s <= num_cus / 8; s++)
+        if (nk % (2 * s) == 0 && nk / s >= 6) best = s;
+    return best;
+}
+
 hipError_t launch_gemm_fp8_fast(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
-    dim3            grid((p.M / FBM) * (p.N / FBN), (unsigned) nb, 1);
+    dim3            grid((p.M / FBM) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {
         case 0: return launch_fmt<0>(p, grid, s);

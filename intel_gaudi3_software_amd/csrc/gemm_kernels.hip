@@ -100,6 +100,7 @@ size_t gemm_workspace_bytes(const GemmProblem& p)
 
 int gemm_pick_split_k(const GemmProblem& p, int num_cus)
 {
+    if (const int fast = gemm_fast_pick_split_k(p, num_cus)) return fast; // the large-tile kernel takes this problem
     // split the reduction only when the output tiles cannot fill the chip and the reduction is long
     const long long tiles = (long long) ((p.M + TILE - 1) / TILE) * ((p.N + TILE - 1) / TILE) * p.batch[0] * p.batch[1] * p.batch[2];
     const int       es = (p.dtype == DT_BF16) ? 2 : (p.dtype == DT_FP32 ? 4 : 1);
@@ -115,26 +116,30 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     if (p.M <= 0 || p.N <= 0 || nb <= 0) return hipSuccess;
-    if (gemm_fp8_fast_applicable(p)) return launch_gemm_fp8_fast(p, s);
-    const int tiles = ((p.M + TILE - 1) / TILE) * ((p.N + TILE - 1) / TILE);
-    dim3      grid(tiles, (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
-    switch (p.dtype)
+    hipError_t e;
+    if (gemm_fp8_fast_applicable(p)) e = launch_gemm_fp8_fast(p, s);
+    else
     {
-        case DT_BF16: launch_gemm_bf16(p, grid, s); break;
-        case DT_FP32: launch_gemm_fp32(p, grid, s); break;
-        case DT_FP8_143:
-        case DT_FP8_152:
-            switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
-            {
-                case 0: launch_gemm_fp8_00(p, grid, s); break;
-                case 1: launch_gemm_fp8_10(p, grid, s); break;
-                case 2: launch_gemm_fp8_01(p, grid, s); break;
-                default: launch_gemm_fp8_11(p, grid, s); break;
-            }
-            break;
-        default: return hipErrorInvalidValue;
+        const int tiles = ((p.M + TILE - 1) / TILE) * ((p.N + TILE - 1) / TILE);
+        dim3      grid(tiles, (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+        switch (p.dtype)
+        {
+            case DT_BF16: launch_gemm_bf16(p, grid, s); break;
+            case DT_FP32: launch_gemm_fp32(p, grid, s); break;
+            case DT_FP8_143:
+            case DT_FP8_152:
+                switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
+                {
+                    case 0: launch_gemm_fp8_00(p, grid, s); break;
+                    case 1: launch_gemm_fp8_10(p, grid, s); break;
+                    case 2: launch_gemm_fp8_01(p, grid, s); break;
+                    default: launch_gemm_fp8_11(p, grid, s); break;
+                }
+                break;
+            default: return hipErrorInvalidValue;
+        }
+        e = hipGetLastError();
     }
-    hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (p.split_k > 1)
     {

@@ -279,3 +279,38 @@ def test_fp8_fast_kernel_epilogue_overflow_takes_exact_conversion(calc, orc, cli
     got = out.cpu().numpy().view(np.uint16)
     assert np.array_equal(got, want)
     assert (np.any((want & 0x7FFF) == 0x7F7F) if clip else np.any((want & 0x7FFF) == 0x7F80))
+
+
+@pytest.mark.parametrize("op", [abi.OP_AB, abi.OP_ABT])
+def test_bf16_fast_kernel_vs_oracle(calc, orc, op):
+    """bf16 shapes that take the large-tile kernel (M, N multiples of 256, K multiple of 64 and >= 192), both B layouts,
+    batch of 2 with B broadcast; fp32 accumulators against the oracle."""
+    got, want = _run_both(calc, orc, op, 256, 512, 320, abi.BF16, abi.BF16, 0, 0, 0, 0, batch=(2, 1, 1), bcast_b=True, seed=80 + op,
+                          device=True)
+    assert rel_frobenius(got, want) <= 2e-3
+    assert rel_frobenius(got, want) <= 1e-4
+
+
+@pytest.mark.parametrize("b_kc", [False, True])
+def test_bf16_fast_kernel_every_k_position(calc, orc, b_kc):
+    """One-hot bf16 operands walk a single product through every k position and tile coordinate of the large-tile kernel:
+    the k order of the transposing reads of an n-contiguous B must match the k-contiguous reads of A."""
+    import torch
+    from helpers import to_bf16_bits
+    M, N, K = 256, 256, 384
+    a = np.zeros((M, K), np.float32)
+    b = np.zeros((K, N), np.float32)
+    rng = np.random.default_rng(5)
+    perm_m = rng.permutation(M)
+    for k in range(K):
+        a[perm_m[k % M], k] = 1.0 + (k % 5)
+        b[k, (k * 11 + 2) % N] = 2.0 if k % 2 else 1.0
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    bmat = b.T.copy() if b_kc else b
+    ta = torch.from_numpy(to_bf16_bits(a.ravel()).view(np.int16)).cuda()
+    tb = torch.from_numpy(to_bf16_bits(bmat.ravel()).view(np.int16)).cuda()
+    out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, abi.BF16, ta),
+                     MmeSimTensor([K, N] if b_kc else [N, K], 2, abi.BF16, tb), abi.OP_ABT if b_kc else abi.OP_AB)
+    calc.synchronize()
+    assert np.array_equal(out.cpu().numpy().reshape(M, N).astype(np.float64), want)
