@@ -114,14 +114,20 @@ __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int w
 
 // ES = 1: fp8 (FMT selects e4m3 / e5m2 per operand), ES = 2: bf16.  Everything up to the matrix-core instruction is
 // byte-based and shared: a stage is 64 bytes of k per row for both.
-template<int ES, int FMT, bool B_KC>
+// GATHER: A is a convolution view with pixels along f (im2col addressing of mme/mme_reference/im2col.cpp:134-172 for the
+// forward pass, its gather-form inverse for dedx): row r of the tile is a pixel, a 64-byte stage is a run of channels
+// of one filter tap, so a request's address is (pixel's offset for tap 0) + (the tap's uniform offset) + channel, or a
+// page of zeros where the tap falls outside the source tensor.  B may then be a tapped weight view (dedx).
+__device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
+
+template<int ES, int FMT, bool B_KC, bool GATHER = false>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     if (g.skip_flag && ((*g.skip_flag != 0u) == (g.skip_if != 0))) return;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
-    const int tiles_n = g.N / FBN, tiles_m = g.M / FBM;
+    const int tiles_n = g.N / FBN, tiles_m = (g.M + FBM - 1) / FBM;
     int       tm, tn;
     {
         const int b = blockIdx.x, T = tiles_m * tiles_n;
@@ -167,6 +173,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     for (int u = 0; u < 2; u++)
     {
         const int t = wave * 2 + u;
+        if constexpr (!GATHER)
         {
             const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
             ga[u] = A + (size_t) (m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
@@ -176,6 +183,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
             gb[u] = B + (size_t) (n0 + r) * ldb + c * 16 + (size_t) kt_begin * FBK;
         }
+        else if (GATHER && g.B.kind == VIEW_TAPPED)
+            gb[u] = nullptr; // (tapped weights are k-contiguous: B_KC)
         else if (ES == 1)
         {
             const int k = t * 4 + (lane >> 4), p = lane & 15, cb = (p - 2 * (k & 7)) & 15;
@@ -187,13 +196,87 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             gb[u] = B + (size_t) (k + kt_begin * (FBK / 2)) * ldb + n0 * 2 + chunk * 16;
         }
     }
+    // ---- GATHER: per-row tap masks and the running (tap, channel) position of the stage being requested ----------------
+    uint32_t  tap_ok[2] = {0, 0};      // bit t: tap t of this lane's row (request slot u) reads inside the source tensor
+    int       g_tap = 0, g_ch = 0;     // uniform: tap and first channel of the next stage to request
+    int       g_t[3] = {0, 0, 0};      // g_tap as (s, r, q)
+    long long g_delta_a = 0, g_delta_b = 0; // uniform byte offsets of that stage: tap offset + channel
+    const int stage_ch = FBK / ES;     // channels per stage
+    auto      gather_offsets = [&]() __attribute__((always_inline))
+    {
+        long long d = 0;
+#pragma unroll
+        for (int q = 0; q < 3; q++) d += (long long) g_t[q] * g.A.dil[q] * g.A.src_stride[q];
+        g_delta_a = ((g.A.gather_y ? -d : d) + g_ch) * ES;
+        g_delta_b = ((long long) g_tap * g.B.tap_stride + g_ch) * ES;
+    };
+    auto gather_advance = [&]() __attribute__((always_inline))
+    {
+        g_ch += stage_ch;
+        if (g_ch >= g.A.nch)
+        {
+            g_ch = 0;
+            g_tap++;
+            if (++g_t[0] == g.A.ktap[0])
+            {
+                g_t[0] = 0;
+                if (++g_t[1] == g.A.ktap[1])
+                {
+                    g_t[1] = 0;
+                    g_t[2]++;
+                }
+            }
+        }
+        gather_offsets();
+    };
+    if constexpr (GATHER)
+    {
+        const int ntaps = g.A.ktap[0] * g.A.ktap[1] * g.A.ktap[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+        {
+            const int r = (wave * 2 + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
+            const int pix = min(m0 + r, g.M - 1);
+            const PixelPos pp = decode_pixel(g.A, pix);
+            long long      off0 = 0;
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+                off0 += (long long) (g.A.gather_y ? pp.c[d] + g.A.pad[d] : pp.c[d] * g.A.cstride[d] - g.A.pad[d]) * g.A.src_stride[d];
+            ga[u] = A + off0 * ES + c * 16;
+            if (m0 + r < g.M)
+                for (int t = 0; t < ntaps; t++) tap_ok[u] |= (conv_offset(g.A, pp, t) >= 0 ? 1u : 0u) << t;
+            if (g.B.kind == VIEW_TAPPED) gb[u] = B + (size_t) (n0 + r) * ldb + c * 16;
+        }
+        // first stage of this workgroup's k range
+        const int k0 = kt_begin * stage_ch;
+        g_tap = k0 / g.A.nch;
+        g_ch = k0 - g_tap * g.A.nch;
+        g_t[0] = g_tap % g.A.ktap[0];
+        g_t[1] = (g_tap / g.A.ktap[0]) % g.A.ktap[1];
+        g_t[2] = g_tap / (g.A.ktap[0] * g.A.ktap[1]);
+        gather_offsets();
+    }
     auto issue_a = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
-        dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+        if constexpr (GATHER)
+        {
+            const bool     ok = (tap_ok[u] >> g_tap) & 1u;
+            const uint8_t* src = ok ? ga[u] + g_delta_a : (const uint8_t*) gf_zero_page;
+            dma16(src, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+        }
+        else
+            dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
     };
     auto issue_b = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
+        if (GATHER && g.B.kind == VIEW_TAPPED)
+        {
+            dma16(gb[u] + g_delta_b, lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
+            if (u == 1) gather_advance(); // the stage's last request
+            return;
+        }
         dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
+        if (GATHER && u == 1) gather_advance();
     };
     auto read_b = [&](Frags & f, int j, const char* st) __attribute__((always_inline))
     {
@@ -352,7 +435,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             {
                 float val[16];
                 gather(i, j, val);
-                store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
+                if (!GATHER || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
             }
     };
     typedef float    e_v4f __attribute__((ext_vector_type(4)));
@@ -369,7 +452,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #pragma unroll
             for (int j = 0; j < 2; j++)
             {
-                e_v4f* o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
+                e_v4f*     o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
+                const bool row_ok = !GATHER || m0 + wm * 128 + i * 32 + (lane & 31) < g.M;
 #pragma unroll
                 for (int q = 0; q < 2; q++)
                 {
@@ -382,8 +466,11 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                         lo4[r] = __uint_as_float(sw[0]);
                         hi4[r] = __uint_as_float(sw[1]);
                     }
-                    o[2 * q] = e_v4f {lo4[0], lo4[1], lo4[2], lo4[3]};
-                    o[2 * q + 1] = e_v4f {hi4[0], hi4[1], hi4[2], hi4[3]};
+                    if (row_ok)
+                    {
+                        o[2 * q] = e_v4f {lo4[0], lo4[1], lo4[2], lo4[3]};
+                        o[2 * q + 1] = e_v4f {hi4[0], hi4[1], hi4[2], hi4[3]};
+                    }
                 }
             }
     }
@@ -477,7 +564,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                     float x = val[c];
                     if (has_alpha) x *= alpha;
                     if (col_exp) x *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
-                    store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
+                    if (!GATHER || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
                 }
             }
     }
@@ -496,6 +583,30 @@ __global__ __launch_bounds__(512) void gemm_bf16_fast_kernel(GemmProblem g_by_va
 {
     (void) g_by_value;
     gemm_fast_body<2, 0, B_KC>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+}
+
+template<bool B_KC>
+__global__ __launch_bounds__(512) void conv_bf16_fast_kernel(GemmProblem g_by_value)
+{
+    (void) g_by_value;
+    gemm_fast_body<2, 0, B_KC, true>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+}
+
+hipError_t launch_conv_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
+{
+    static bool attr_done[2] = {false, false};
+    const bool  bkc = p.B.k_contig != 0;
+    const void* fn = bkc ? (const void*) conv_bf16_fast_kernel<true> : (const void*) conv_bf16_fast_kernel<false>;
+    if (!attr_done[bkc])
+    {
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, FNST * FSTAGE);
+        if (e != hipSuccess) return e;
+        attr_done[bkc] = true;
+    }
+    if (bkc) hipLaunchKernelGGL((conv_bf16_fast_kernel<true>), grid, dim3(512), FNST * FSTAGE, s, p);
+    else
+        hipLaunchKernelGGL((conv_bf16_fast_kernel<false>), grid, dim3(512), FNST * FSTAGE, s, p);
+    return hipGetLastError();
 }
 
 hipError_t launch_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
@@ -538,9 +649,23 @@ bool gemm_fp8_fast_applicable(const GemmProblem& p)
 {
     if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152 || p.dtype == DT_BF16)) return false;
     const int es = p.dtype == DT_BF16 ? 2 : 1;
-    if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN) return false;
+    const bool gather = p.A.kind == VIEW_CONV;
+    if (gather)
+    {
+        // pixels along f, bf16, whole 64-byte stages inside one tap, at most 32 taps; the gather form of col2im only
+        // with unit strides; weights plain or tapped (k-contiguous, same channel count)
+        if (p.dtype != DT_BF16 || !p.A.pix_is_f) return false;
+        if (p.A.nch % (FBK / es) || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
+        for (int d = 0; d < 4; d++)
+            if (p.A.gather_y && p.A.cstride[d] != 1) return false;
+        if (p.B.kind == VIEW_TAPPED && (!p.B.k_contig || p.B.nch != p.A.nch || p.B.stride_k != 1)) return false;
+        if (p.B.kind != VIEW_TAPPED && p.B.kind != VIEW_PLAIN) return false;
+        if (p.batch[0] * p.batch[1] * p.batch[2] != 1) return false;
+    }
+    else if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN)
+        return false;
     if (!p.A.k_contig || !p.A.vec_ok || !p.B.vec_ok) return false;
-    if (p.M % FBM || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
+    if ((!gather && p.M % FBM) || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
     if (p.split_k > 1)
     {
         // every slice an even number of stages, at least 6
@@ -564,7 +689,7 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
     GemmProblem q = p;
     q.split_k = 1;
     if (!gemm_fp8_fast_applicable(q)) return 0;
-    const long long tiles = (long long) (p.M / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
+    const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
     const int       nk = p.K * (p.dtype == DT_BF16 ? 2 : 1) / FBK;
     int             best = 1;
     // Splitting pays only while the tiles leave most of the chip idle: each slice costs a pass of the fp32 output through
@@ -577,7 +702,8 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
 hipError_t launch_gemm_fp8_fast(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
-    dim3            grid((p.M / FBM) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    dim3            grid(((p.M + FBM - 1) / FBM) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    if (p.A.kind == VIEW_CONV) return launch_conv_bf16(p, grid, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {

@@ -158,3 +158,59 @@ def test_conv_fwd_fast_path_special_values(calc, orc, relu, clip):
     want16 = np.zeros(n, np.uint16)
     assert orc.orc_cast_from_fp32(want16.ctypes.data, abi.BF16, 0, 0, got.ctypes.data, n, 0, None, 0, int(relu), 0, int(clip), 0, 0) == 0
     assert np.array_equal(out.cpu().numpy().view(np.uint16), want16)
+
+
+# shapes that take the large-tile kernel with the gather on its load side: bf16, 256 output columns, channel counts that
+# are multiples of 32; ragged pixel counts, dilation, a strided forward pass, a 1 x 1 filter
+GATHER_CASES = [
+    (256, 256, 9, 7, 1, 2, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),
+    (64, 256, 11, 6, 1, 1, 3, 3, 1, (2, 2, 0), (1, 1, 1), (2, 2, 1), 2),
+    (256, 256, 8, 8, 1, 1, 1, 1, 1, (0, 0, 0), (1, 1, 1), (1, 1, 1), 2),
+]
+
+
+@pytest.mark.parametrize("case", GATHER_CASES)
+@pytest.mark.parametrize("op", [abi.OP_FWD, abi.OP_DEDX])
+def test_conv_large_tile_gather_vs_oracle(calc, orc, case, op):
+    if op == abi.OP_DEDX and case[0] != 256:
+        pytest.skip("dedx has C output columns: only C = 256 takes the large-tile kernel")
+    if case[6] == 1 and op == abi.OP_FWD:
+        pass  # K * taps = 256 channels: 8 stages
+    got, want = _run(calc, orc, case, abi.BF16, 0, op, device=True)
+    assert rel_frobenius(got, want) <= TOL[abi.BF16]
+    assert rel_frobenius(got, want) <= 1e-4
+
+
+def test_conv_large_tile_strided_forward_vs_oracle(calc, orc):
+    case = (64, 256, 13, 9, 1, 2, 3, 3, 1, (1, 1, 0), (2, 2, 1), (1, 1, 1), 2)
+    got, want = _run(calc, orc, case, abi.BF16, 0, abi.OP_FWD, device=True)
+    assert rel_frobenius(got, want) <= 1e-4
+
+
+def test_conv_adjoint_identities_256_channels(calc, orc):
+    """<dY, fwd(X, W)> = <dedx(dY, W), X> = <dedw(X, dY), W> with 256 channels: fwd and dedx on the large-tile kernel (four
+    tiles, the last one ragged), dedw on the general kernel."""
+    import torch
+    rng = np.random.default_rng(78)
+    C, K, W, H, B = 256, 256, 14, 14, 4
+    xs, ws, ys = [C, W, H, 1, B], [K, C, 3, 3, 1], [K, W, H, 1, B]
+    from helpers import bf16_bits_to_f32, to_bf16_bits
+    x = to_bf16_bits(rng.standard_normal(int(np.prod(xs))))
+    w = to_bf16_bits(rng.standard_normal(int(np.prod(ws))) * 0.05)
+    dy = to_bf16_bits(rng.standard_normal(int(np.prod(ys))))
+    conv = lambda a: torch.from_numpy(a.view(np.int16)).cuda()
+    tx, tw, ty = conv(x), conv(w), conv(dy)
+    X, Wt, Y = MmeSimTensor(xs, 5, abi.BF16, tx), MmeSimTensor(ws, 5, abi.BF16, tw), MmeSimTensor(ys, 5, abi.BF16, ty)
+    cp = ConvolutionParams(2, [1, 1, 0, 0], [1, 1, 1, 1], [1, 1, 1, 1])
+    f = torch.zeros(int(np.prod(ys)), dtype=torch.float32, device="cuda")
+    gx = torch.zeros(int(np.prod(xs)), dtype=torch.float32, device="cuda")
+    gw = torch.zeros(int(np.prod(ws)), dtype=torch.float32, device="cuda")
+    calc.doConvolution(MmeSimTensor(ys, 5, abi.FP32, f), X, Wt, Y, cp, abi.OP_FWD)
+    calc.doConvolution(MmeSimTensor(xs, 5, abi.FP32, gx), X, Wt, Y, cp, abi.OP_DEDX)
+    calc.doConvolution(MmeSimTensor(ws, 5, abi.FP32, gw), X, Wt, Y, cp, abi.OP_DEDW)
+    calc.synchronize()
+    xf, wf, yf = (bf16_bits_to_f32(v).astype(np.float64) for v in (x, w, dy))
+    s_f = np.dot(yf, f.cpu().numpy().astype(np.float64))
+    s_x = np.dot(xf, gx.cpu().numpy().astype(np.float64))
+    s_w = np.dot(wf, gw.cpu().numpy().astype(np.float64))
+    assert abs(s_f - s_x) <= 1e-4 * abs(s_f) and abs(s_f - s_w) <= 1e-4 * abs(s_f)
