@@ -102,6 +102,25 @@ __device__ __forceinline__ void read_b_tr16(Frags& f, int j, const char* st, int
     f.b[j] = u.v;
 }
 
+// bf16, A stored f-contiguous: the same stage layout and reads as an n-contiguous B, over the wavefront's 128 rows
+__device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int wm, int lane)
+{
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wm * 8 + i * 2 + (g & 1);
+    union
+    {
+        v4s h4[4];
+        v8i v;
+    } u;
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+    {
+        const int k = 16 * h + 4 * tt + (q >> 2);
+        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + k * 512 + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
+    }
+    f.a[i] = u.v;
+}
+
 // B stored k-contiguous (the "abt" form): same layout and reads as A
 __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int wn, int lane)
 {
@@ -120,9 +139,17 @@ __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int w
 // page of zeros where the tap falls outside the source tensor.  B may then be a tapped weight view (dedx).
 __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 
-template<int ES, int FMT, bool B_KC, bool GATHER = false>
+//
+// AMODE says how operand A is addressed: 0 plain, k contiguous; 1 convolution view with pixels along f (GATHER above);
+// 2 plain, f contiguous (the "atb" forms; bf16 only: the stage then holds 32 k-rows x 256 f like an n-contiguous B and is
+// read with ds_read_b64_tr_b16); 3 convolution view with pixels along k (dedw: f = tap * channels + channel is fixed per
+// lane, the pixel advances by 32 per stage and is decoded incrementally).
+template<int ES, int FMT, bool B_KC, int AMODE = 0>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
+    constexpr bool GATHER = AMODE == 1;           // tap masks + uniform tap offsets
+    constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3; // the last row tile may be partial
+    constexpr bool A_KC = AMODE < 2;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     if (g.skip_flag && ((*g.skip_flag != 0u) == (g.skip_if != 0))) return;
 
@@ -150,7 +177,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     const long long a_off = b0 * g.A.batch_stride[0] + b1 * g.A.batch_stride[1] + b2 * g.A.batch_stride[2];
     const long long b_off = b0 * g.B.batch_stride[0] + b1 * g.B.batch_stride[1] + b2 * g.B.batch_stride[2];
     const int       m0 = tm * FBM, n0 = tn * FBN;
-    const long long lda = g.A.stride_f * ES; // bytes
+    const long long lda = (A_KC ? g.A.stride_f : g.A.stride_k) * ES; // bytes between rows of the staged A tile
     const long long ldb = (B_KC ? g.B.stride_f : g.B.stride_k) * ES;
     const uint8_t*  A = (const uint8_t*) g.A.base + a_off * ES;
     const uint8_t*  B = (const uint8_t*) g.B.base + b_off * ES;
@@ -173,10 +200,15 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     for (int u = 0; u < 2; u++)
     {
         const int t = wave * 2 + u;
-        if constexpr (!GATHER)
+        if constexpr (AMODE == 0)
         {
             const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
             ga[u] = A + (size_t) (m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
+        }
+        if constexpr (AMODE == 2)
+        {
+            const int k = t * 2 + (lane >> 5), p = lane & 31, chunk = p ^ ((k & 3) << 1);
+            ga[u] = A + (size_t) (k + kt_begin * (FBK / 2)) * lda + m0 * 2 + chunk * 16;
         }
         if (B_KC)
         {
@@ -256,9 +288,63 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         g_t[2] = g_tap / (g.A.ktap[0] * g.A.ktap[1]);
         gather_offsets();
     }
+    // ---- AMODE 3: this lane's (tap, channel) per request slot and the pixel of the next stage to request -----------------
+    int       w_pc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}}; // pixel coordinates (dims 1..4 of the tensor that enumerates pixels)
+    int       w_t[2][3] = {{0, 0, 0}, {0, 0, 0}};        // tap as (s, r, q)
+    long long w_ch[2] = {0, 0};                          // channel byte offset, < 0: f beyond M
+    float     w_rcp[3] = {0.0f, 0.0f, 0.0f};             // 1 / grid[d]
+    if constexpr (AMODE == 3)
+    {
+#pragma unroll
+        for (int d = 0; d < 3; d++) w_rcp[d] = __builtin_amdgcn_rcpf((float) g.A.grid[d]);
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+        {
+            const int kr = (wave * 2 + u) * 2 + (lane >> 5), chunk = (lane & 31) ^ ((kr & 3) << 1);
+            const int f = m0 + chunk * 8, tap = f / g.A.nch;
+            w_ch[u] = f < g.M ? (long long) (f - tap * g.A.nch) * 2 : -1;
+            w_t[u][0] = tap % g.A.ktap[0];
+            w_t[u][1] = (tap / g.A.ktap[0]) % g.A.ktap[1];
+            w_t[u][2] = tap / (g.A.ktap[0] * g.A.ktap[1]);
+            const PixelPos pp = decode_pixel(g.A, kt_begin * (FBK / 2) + kr);
+#pragma unroll
+            for (int d = 0; d < 4; d++) w_pc[u][d] = pp.c[d];
+        }
+    }
     auto issue_a = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
-        if constexpr (GATHER)
+        if constexpr (AMODE == 3)
+        {
+            // x[pos(pixel, tap)][channel .. + 7], or zeros where the tap falls into the padding
+            long long off = w_ch[u];
+            bool      ok = off >= 0;
+#pragma unroll
+            for (int d = 0; d < 4; d++)
+            {
+                const int pos = w_pc[u][d] * g.A.cstride[d] + (d < 3 ? w_t[u][d] * g.A.dil[d] : 0) - g.A.pad[d];
+                ok = ok && pos >= 0 && pos < g.A.src[d];
+                off += (long long) pos * g.A.src_stride[d] * 2;
+            }
+            const uint8_t* src = ok ? A + off : (const uint8_t*) gf_zero_page;
+            dma16(src, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+            // next stage: 32 pixels further
+            int carry = 32;
+#pragma unroll
+            for (int d = 0; d < 3; d++)
+            {
+                // v / grid[d] for small non-negative v: float estimate, corrected by one
+                const int v = w_pc[u][d] + carry, gd = g.A.grid[d];
+                int       q = (int) ((float) v * w_rcp[d]);
+                const int r = v - q * gd;
+                q += (r >= gd) - (r < 0);
+                carry = q;
+                w_pc[u][d] = v - q * gd;
+            }
+            w_pc[u][3] += carry;
+        }
+        else if constexpr (AMODE == 2)
+            dma16(ga[u] + (size_t) stage * (FBK / ES) * lda, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+        else if constexpr (GATHER)
         {
             const bool     ok = (tap_ok[u] >> g_tap) & 1u;
             const uint8_t* src = ok ? ga[u] + g_delta_a : (const uint8_t*) gf_zero_page;
@@ -299,9 +385,15 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     // s_waitcnt immediate (gfx9): vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
     __builtin_amdgcn_s_waitcnt(0x0F78); // vmcnt(8): stage 0 has landed
     __syncthreads();
+    auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
+    {
+        if constexpr (A_KC) read_a(fr, i, st, wm, lane);
+        else
+            read_a_tr16(fr, i, st, wm, lane);
+    };
     Frags f;
 #pragma unroll
-    for (int i = 0; i < 4; i++) read_a(f, i, lds, wm, lane);
+    for (int i = 0; i < 4; i++) read_a_any(f, i, lds);
 #pragma unroll
     for (int j = 0; j < 2; j++) read_b(f, j, lds);
 
@@ -324,7 +416,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     };
 #define MMA(i, j) mma(i, j)
 #define RA(i) \
-    if (RN) read_a(f, i, st, wm, lane);
+    if (RN) read_a_any(f, i, st);
 #define RB(j) \
     if (RN) read_b(f, j, st);
 #define LA(u) \
@@ -435,7 +527,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             {
                 float val[16];
                 gather(i, j, val);
-                if (!GATHER || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
+                if (!RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
             }
     };
     typedef float    e_v4f __attribute__((ext_vector_type(4)));
@@ -453,7 +545,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             for (int j = 0; j < 2; j++)
             {
                 e_v4f*     o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
-                const bool row_ok = !GATHER || m0 + wm * 128 + i * 32 + (lane & 31) < g.M;
+                const bool row_ok = !RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M;
 #pragma unroll
                 for (int q = 0; q < 2; q++)
                 {
@@ -564,7 +656,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                     float x = val[c];
                     if (has_alpha) x *= alpha;
                     if (col_exp) x *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
-                    if (!GATHER || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
+                    if (!RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
                 }
             }
     }
@@ -578,18 +670,25 @@ __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_val
     gemm_fast_body<1, FMT, B_KC>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
 }
 
-template<bool B_KC>
+template<bool B_KC, bool A_KC>
 __global__ __launch_bounds__(512) void gemm_bf16_fast_kernel(GemmProblem g_by_value)
 {
     (void) g_by_value;
-    gemm_fast_body<2, 0, B_KC>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+    gemm_fast_body<2, 0, B_KC, A_KC ? 0 : 2>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+}
+
+// dedw: pixels along k for both operands, dY plain and n-contiguous
+__global__ __launch_bounds__(512) void conv_dedw_bf16_fast_kernel(GemmProblem g_by_value)
+{
+    (void) g_by_value;
+    gemm_fast_body<2, 0, false, 3>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
 }
 
 template<bool B_KC>
 __global__ __launch_bounds__(512) void conv_bf16_fast_kernel(GemmProblem g_by_value)
 {
     (void) g_by_value;
-    gemm_fast_body<2, 0, B_KC, true>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+    gemm_fast_body<2, 0, B_KC, 1>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
 }
 
 hipError_t launch_conv_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
@@ -609,21 +708,28 @@ hipError_t launch_conv_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
     return hipGetLastError();
 }
 
+template<class K>
+hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s)
+{
+    if (!attr_done)
+    {
+        hipError_t e = hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FNST * FSTAGE);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(512), FNST * FSTAGE, s, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
 {
-    static bool attr_done[2] = {false, false};
-    const bool  bkc = p.B.k_contig != 0;
-    const void* fn = bkc ? (const void*) gemm_bf16_fast_kernel<true> : (const void*) gemm_bf16_fast_kernel<false>;
-    if (!attr_done[bkc])
-    {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, FNST * FSTAGE);
-        if (e != hipSuccess) return e;
-        attr_done[bkc] = true;
-    }
-    if (bkc) hipLaunchKernelGGL((gemm_bf16_fast_kernel<true>), grid, dim3(512), FNST * FSTAGE, s, p);
-    else
-        hipLaunchKernelGGL((gemm_bf16_fast_kernel<false>), grid, dim3(512), FNST * FSTAGE, s, p);
-    return hipGetLastError();
+    static bool attr_done[5] = {false, false, false, false, false};
+    const bool  bkc = p.B.k_contig != 0, akc = p.A.k_contig != 0;
+    if (p.A.kind == VIEW_CONV && !p.A.pix_is_f) return launch_fast(conv_dedw_bf16_fast_kernel, attr_done[4], p, grid, s);
+    if (akc) return bkc ? launch_fast(gemm_bf16_fast_kernel<true, true>, attr_done[0], p, grid, s)
+                        : launch_fast(gemm_bf16_fast_kernel<false, true>, attr_done[1], p, grid, s);
+    return bkc ? launch_fast(gemm_bf16_fast_kernel<true, false>, attr_done[2], p, grid, s)
+               : launch_fast(gemm_bf16_fast_kernel<false, false>, attr_done[3], p, grid, s);
 }
 
 template<int FMT>
@@ -652,19 +758,30 @@ bool gemm_fp8_fast_applicable(const GemmProblem& p)
     const bool gather = p.A.kind == VIEW_CONV;
     if (gather)
     {
-        // pixels along f, bf16, whole 64-byte stages inside one tap, at most 32 taps; the gather form of col2im only
-        // with unit strides; weights plain or tapped (k-contiguous, same channel count)
-        if (p.dtype != DT_BF16 || !p.A.pix_is_f) return false;
-        if (p.A.nch % (FBK / es) || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
-        for (int d = 0; d < 4; d++)
-            if (p.A.gather_y && p.A.cstride[d] != 1) return false;
-        if (p.B.kind == VIEW_TAPPED && (!p.B.k_contig || p.B.nch != p.A.nch || p.B.stride_k != 1)) return false;
-        if (p.B.kind != VIEW_TAPPED && p.B.kind != VIEW_PLAIN) return false;
+        // bf16, at most 32 taps, one problem per launch
+        if (p.dtype != DT_BF16 || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
         if (p.batch[0] * p.batch[1] * p.batch[2] != 1) return false;
+        if (p.A.pix_is_f)
+        {
+            // fwd / dedx: whole 64-byte stages inside one tap; the gather form of col2im only with unit strides; weights
+            // plain or tapped (k-contiguous, same channel count)
+            if (p.A.nch % (FBK / es)) return false;
+            for (int d = 0; d < 4; d++)
+                if (p.A.gather_y && p.A.cstride[d] != 1) return false;
+            if (p.B.kind == VIEW_TAPPED && (!p.B.k_contig || p.B.nch != p.A.nch || p.B.stride_k != 1)) return false;
+            if (p.B.kind != VIEW_TAPPED && p.B.kind != VIEW_PLAIN) return false;
+        }
+        else
+        {
+            // dedw: 16-byte chunks of channels inside one tap, dY plain with its channels contiguous
+            if (p.A.gather_y || p.A.nch % 8 || p.B.kind != VIEW_PLAIN || p.B.k_contig) return false;
+        }
     }
     else if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN)
         return false;
-    if (!p.A.k_contig || !p.A.vec_ok || !p.B.vec_ok) return false;
+    if (!p.A.vec_ok || !p.B.vec_ok) return false;
+    if (!p.A.k_contig && p.dtype != DT_BF16) return false; // f-contiguous A: bf16 only
+    if (gather && p.A.pix_is_f && !p.A.k_contig) return false;
     if ((!gather && p.M % FBM) || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
     if (p.split_k > 1)
     {
@@ -692,10 +809,22 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
     const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
     const int       nk = p.K * (p.dtype == DT_BF16 ? 2 : 1) / FBK;
     int             best = 1;
-    // Splitting pays only while the tiles leave most of the chip idle: each slice costs a pass of the fp32 output through
-    // the workspace and the reduction kernel.  Every slice keeps an even number of stages, at least 6.
-    for (int s = 2; s <= 4 && tiles * s <= num_cus / 8; s++)
-        if (nk % (2 * s) == 0 && nk / s >= 6) best = s;
+    // Splitting the reduction pays when the tiles leave most of the chip idle and the reduction is long: a slice costs a
+    // pass of the fp32 output through the workspace plus the reduction kernel.  Rough model in microseconds: a stage
+    // takes 0.5, the workspace moves at 4 TB/s, the extra launch costs 6.  Every slice keeps an even number of stages,
+    // at least 6.
+    const double out_bytes = 8.0 * p.M * (double) p.N * p.batch[0] * p.batch[1] * p.batch[2];
+    double       best_t = (double) ((tiles + num_cus - 1) / num_cus) * nk * 0.5;
+    for (int s = 2; s <= 64; s++)
+    {
+        if (nk % (2 * s) || nk / s < 6) continue;
+        const double t = (double) ((tiles * s + num_cus - 1) / num_cus) * (nk / s) * 0.5 + s * out_bytes / 4e6 + 6.0;
+        if (t < 0.8 * best_t)
+        {
+            best_t = t;
+            best = s;
+        }
+    }
     return best;
 }
 
@@ -703,7 +832,7 @@ hipError_t launch_gemm_fp8_fast(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     dim3            grid(((p.M + FBM - 1) / FBM) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
-    if (p.A.kind == VIEW_CONV) return launch_conv_bf16(p, grid, s);
+    if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return launch_conv_bf16(p, grid, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {

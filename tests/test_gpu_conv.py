@@ -181,6 +181,21 @@ def test_conv_large_tile_gather_vs_oracle(calc, orc, case, op):
     assert rel_frobenius(got, want) <= 1e-4
 
 
+# dedw on the large-tile kernel: pixels (the reduction) a multiple of 64 and at least 192, K = 256 output columns
+DEDW_CASES = [
+    (256, 256, 8, 8, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),
+    (64, 256, 16, 8, 1, 2, 3, 3, 1, (2, 2, 0), (1, 1, 1), (2, 2, 1), 2),     # M = 576: ragged row tile, three taps per tile
+    (32, 256, 18, 17, 1, 1, 3, 3, 1, (0, 0, 0), (2, 2, 1), (1, 1, 1), 2),    # strided: 8 x 8 output pixels
+]
+
+
+@pytest.mark.parametrize("case", DEDW_CASES)
+def test_conv_large_tile_dedw_vs_oracle(calc, orc, case):
+    got, want = _run(calc, orc, case, abi.BF16, 0, abi.OP_DEDW, device=True)
+    assert rel_frobenius(got, want) <= TOL[abi.BF16]
+    assert rel_frobenius(got, want) <= 1e-4
+
+
 def test_conv_large_tile_strided_forward_vs_oracle(calc, orc):
     case = (64, 256, 13, 9, 1, 2, 3, 3, 1, (1, 1, 0), (2, 2, 1), (1, 1, 1), 2)
     got, want = _run(calc, orc, case, abi.BF16, 0, abi.OP_FWD, device=True)

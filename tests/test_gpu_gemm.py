@@ -281,9 +281,9 @@ def test_fp8_fast_kernel_epilogue_overflow_takes_exact_conversion(calc, orc, cli
     assert (np.any((want & 0x7FFF) == 0x7F7F) if clip else np.any((want & 0x7FFF) == 0x7F80))
 
 
-@pytest.mark.parametrize("op", [abi.OP_AB, abi.OP_ABT])
+@pytest.mark.parametrize("op", [abi.OP_AB, abi.OP_ABT, abi.OP_ATB, abi.OP_ATBT])
 def test_bf16_fast_kernel_vs_oracle(calc, orc, op):
-    """bf16 shapes that take the large-tile kernel (M, N multiples of 256, K multiple of 64 and >= 192), both B layouts,
+    """bf16 shapes that take the large-tile kernel (M, N multiples of 256, K multiple of 64 and >= 192), all four layouts,
     batch of 2 with B broadcast; fp32 accumulators against the oracle."""
     got, want = _run_both(calc, orc, op, 256, 512, 320, abi.BF16, abi.BF16, 0, 0, 0, 0, batch=(2, 1, 1), bcast_b=True, seed=80 + op,
                           device=True)
