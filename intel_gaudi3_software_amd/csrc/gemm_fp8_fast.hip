@@ -151,7 +151,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3; // the last row tile may be partial
     constexpr bool A_KC = AMODE < 2;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
-    if (g.skip_flag && ((*g.skip_flag != 0u) == (g.skip_if != 0))) return;
+    if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
     const int tiles_n = g.N / FBN, tiles_m = (g.M + FBM - 1) / FBM;

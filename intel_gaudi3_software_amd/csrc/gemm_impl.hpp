@@ -360,7 +360,7 @@ __global__ __launch_bounds__(THREADS) void gemm_kernel(GemmProblem g_by_value)
     KARG GemmProblem& g = *(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr();
     constexpr int BK = STAGE_BYTES / ES;
     __shared__ __attribute__((aligned(16))) char lds[2][2][TILE * LDS_PITCH];
-    if (g.skip_flag && ((*g.skip_flag != 0u) == (g.skip_if != 0))) return;
+    if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
 
     const int tiles_n = (g.N + TILE - 1) / TILE;
     const int tm = blockIdx.x / tiles_n, tn = blockIdx.x % tiles_n;

@@ -19,7 +19,7 @@ __global__ __launch_bounds__(THREADS) void splitk_reduce_kernel(GemmProblem g_by
 {
     (void) g_by_value;
     KARG GemmProblem& g = *(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr();
-    if (g.skip_flag && ((*g.skip_flag != 0u) == (g.skip_if != 0))) return;
+    if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
     const long long mn = (long long) g.M * g.N;
     const long long nb = (long long) g.batch[0] * g.batch[1] * g.batch[2];
     const long long total = mn * nb;
@@ -41,10 +41,10 @@ __global__ __launch_bounds__(THREADS) void splitk_reduce_kernel(GemmProblem g_by
 }
 
 // ---- fp8 helpers --------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(THREADS) void fp8_special_scan_kernel(uint32_t* flag, const uint8_t* data, size_t n, uint32_t exp_mask,
-                                                                   int only_top)
+// exponent-all-ones (only_top: 0x7F / 0xFF) codes in one operand; blocks [first, first + count) of the grid take part
+__device__ __forceinline__ bool fp8_scan_operand(const uint8_t* data, size_t n, uint32_t exp_mask, int only_top, unsigned first, unsigned count)
 {
-    const size_t stride = (size_t) gridDim.x * THREADS;
+    const size_t stride = (size_t) count * THREADS;
     uint32_t     hit = 0;
     const size_t n16 = (((uintptr_t) data & 15u) == 0) ? (n >> 4) : 0;
     const uint4* d16 = reinterpret_cast<const uint4*>(data);
@@ -62,7 +62,7 @@ __global__ __launch_bounds__(THREADS) void fp8_special_scan_kernel(uint32_t* fla
             hit |= (x - 0x01010101u) & ~x & 0x80808080u;
         }
     };
-    for (size_t i = (size_t) blockIdx.x * THREADS + threadIdx.x; i < n16; i += stride)
+    for (size_t i = (size_t) (blockIdx.x - first) * THREADS + threadIdx.x; i < n16; i += stride)
     {
         const uint4 v = d16[i];
         test(v.x);
@@ -70,25 +70,45 @@ __global__ __launch_bounds__(THREADS) void fp8_special_scan_kernel(uint32_t* fla
         test(v.z);
         test(v.w);
     }
-    for (size_t i = (n16 << 4) + (size_t) blockIdx.x * THREADS + threadIdx.x; i < n; i += stride)
+    for (size_t i = (n16 << 4) + (size_t) (blockIdx.x - first) * THREADS + threadIdx.x; i < n; i += stride)
     {
         const uint32_t c = data[i];
         if (only_top ? ((c & 0x7Fu) == 0x7Fu) : ((c & exp_mask) == exp_mask)) hit |= 1u;
     }
-    if (__any(hit != 0u) && (threadIdx.x & 63) == 0) atomicOr(flag, 1u);
+    return hit != 0u;
 }
 
-__global__ __launch_bounds__(THREADS) void fp8_to_bf16_kernel(uint16_t* out, const uint8_t* in, size_t n, int man_bits, int bias, int mode,
-                                                              const uint32_t* run_flag)
+// Both operands in one launch: the first blocks_a blocks scan a, the others b.  A hit stores the call's epoch number;
+// the flag is never reset (epochs only grow), so no separate clearing launch is needed.
+__global__ __launch_bounds__(THREADS) void fp8_special_scan_kernel(uint32_t* flag, uint32_t epoch, const uint8_t* a, size_t na, uint32_t mask_a,
+                                                                   int top_a, unsigned blocks_a, const uint8_t* b, size_t nb, uint32_t mask_b,
+                                                                   int top_b)
 {
-    if (run_flag && *run_flag == 0u) return; // only needed when the scan found codes the hardware formats lack
-    const size_t stride = (size_t) gridDim.x * THREADS;
-    for (size_t i = (size_t) blockIdx.x * THREADS + threadIdx.x; i < n; i += stride)
+    const bool hit = blockIdx.x < blocks_a ? fp8_scan_operand(a, na, mask_a, top_a, 0, blocks_a)
+                                           : fp8_scan_operand(b, nb, mask_b, top_b, blocks_a, gridDim.x - blocks_a);
+    if (__any(hit) && (threadIdx.x & 63) == 0) *(volatile uint32_t*) flag = epoch;
+}
+
+__device__ __forceinline__ void fp8_decode_operand(uint16_t* out, const uint8_t* in, size_t n, int man_bits, int bias, int mode, unsigned first,
+                                                   unsigned count)
+{
+    const size_t stride = (size_t) count * THREADS;
+    for (size_t i = (size_t) (blockIdx.x - first) * THREADS + threadIdx.x; i < n; i += stride)
     {
         // every Gaudi fp8 value (any bias 1..30) is exactly representable in bf16
         const uint32_t f = man_bits == 3 ? fp8_to_fp32<3>(in[i], bias, mode) : fp8_to_fp32<2>(in[i], bias, mode);
         out[i] = (uint16_t) (f >> 16);
     }
+}
+
+__global__ __launch_bounds__(THREADS) void fp8_to_bf16_kernel(uint16_t* out_a, const uint8_t* in_a, size_t na, int man_a, int bias_a, int mode_a,
+                                                              unsigned blocks_a, uint16_t* out_b, const uint8_t* in_b, size_t nb, int man_b,
+                                                              int bias_b, int mode_b, const uint32_t* run_flag, uint32_t epoch)
+{
+    if (run_flag && *run_flag != epoch) return; // only needed when the scan found codes the hardware formats lack
+    if (blockIdx.x < blocks_a) fp8_decode_operand(out_a, in_a, na, man_a, bias_a, mode_a, 0, blocks_a);
+    else
+        fp8_decode_operand(out_b, in_b, nb, man_b, bias_b, mode_b, blocks_a, gridDim.x - blocks_a);
 }
 } // namespace
 
@@ -170,24 +190,37 @@ hipError_t launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s)
     return hipGetLastError();
 }
 
-hipError_t launch_fp8_special_scan(uint32_t* flag, const void* data, size_t n, int man_bits, int mask_kind, hipStream_t s)
+hipError_t launch_fp8_special_scan2(uint32_t* flag, uint32_t epoch, const void* a, size_t na, int man_bits_a, int mask_kind_a, const void* b,
+                                    size_t nb, int man_bits_b, int mask_kind_b, hipStream_t s)
 {
-    if (n == 0) return hipSuccess;
-    const uint32_t exp_mask = man_bits == 3 ? 0x78u : 0x7Cu;
-    size_t         blocks = ((n >> 4) + THREADS - 1) / THREADS + 1;
-    if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(fp8_special_scan_kernel, dim3((unsigned) blocks), dim3(THREADS), 0, s, flag, (const uint8_t*) data, n, exp_mask,
-                       mask_kind);
+    if (mask_kind_a < 0) na = 0;
+    if (mask_kind_b < 0) nb = 0;
+    if (na + nb == 0) return hipSuccess;
+    auto blocks_for = [](size_t n) -> unsigned {
+        if (n == 0) return 0;
+        size_t blocks = ((n >> 4) + THREADS - 1) / THREADS + 1;
+        return (unsigned) (blocks > 1024 ? 1024 : blocks);
+    };
+    const unsigned ba = blocks_for(na), bb = blocks_for(nb);
+    hipLaunchKernelGGL(fp8_special_scan_kernel, dim3(ba + bb), dim3(THREADS), 0, s, flag, epoch, (const uint8_t*) a, na,
+                       man_bits_a == 3 ? 0x78u : 0x7Cu, mask_kind_a > 0 ? 1 : 0, ba, (const uint8_t*) b, nb, man_bits_b == 3 ? 0x78u : 0x7Cu,
+                       mask_kind_b > 0 ? 1 : 0);
     return hipGetLastError();
 }
 
-hipError_t launch_fp8_to_bf16(uint16_t* out, const uint8_t* in, size_t n, int man_bits, int bias, int mode, const uint32_t* run_flag,
-                              hipStream_t s)
+hipError_t launch_fp8_to_bf16_2(uint16_t* out_a, const uint8_t* in_a, size_t na, int man_bits_a, int bias_a, int mode_a, uint16_t* out_b,
+                                const uint8_t* in_b, size_t nb, int man_bits_b, int bias_b, int mode_b, const uint32_t* run_flag, uint32_t epoch,
+                                hipStream_t s)
 {
-    if (n == 0) return hipSuccess;
-    size_t blocks = (n + THREADS - 1) / THREADS;
-    if (blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(fp8_to_bf16_kernel, dim3((unsigned) blocks), dim3(THREADS), 0, s, out, in, n, man_bits, bias, mode, run_flag);
+    if (na + nb == 0) return hipSuccess;
+    auto blocks_for = [](size_t n) -> unsigned {
+        if (n == 0) return 0;
+        size_t blocks = (n + 8 * THREADS - 1) / (8 * THREADS);
+        return (unsigned) (blocks > 1024 ? 1024 : blocks);
+    };
+    const unsigned ba = blocks_for(na), bb = blocks_for(nb);
+    hipLaunchKernelGGL(fp8_to_bf16_kernel, dim3(ba + bb), dim3(THREADS), 0, s, out_a, in_a, na, man_bits_a, bias_a, mode_a, ba, out_b, in_b, nb,
+                       man_bits_b, bias_b, mode_b, run_flag, epoch);
     return hipGetLastError();
 }
 

@@ -54,7 +54,8 @@ struct mme_hip_calc
     std::string           error;
     DeviceBuffer          split_ws;  // split-k partial sums
     DeviceBuffer          decode_ws; // bf16 copies of fp8 operands the hardware formats cannot express
-    DeviceBuffer          flag;      // one 32-bit cell: "operands hold codes the hardware formats lack"
+    DeviceBuffer          flag;      // one 32-bit cell: epoch number of the latest call whose operands held codes the hardware formats lack
+    uint32_t              specials_epoch = 0; // epoch number of the latest call that scanned
     int                   fp8_specials_policy = 0;
 };
 
@@ -244,7 +245,11 @@ void set_plain_view(OperandView& v, const void* base, long long stride_f, long l
 
 int ensure_flag(mme_hip_handle h)
 {
-    if (!h->flag.p) HIP_TRY(h, h->flag.reserve(256));
+    if (!h->flag.p)
+    {
+        HIP_TRY(h, h->flag.reserve(256));
+        HIP_TRY(h, launch_fill_u32((uint32_t*) h->flag.p, 0u, 64, h->stream)); // epoch numbers start at 1
+    }
     return MME_HIP_OK;
 }
 
@@ -290,16 +295,13 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     }
     // scan -> flag; native kernel runs when flag == 0; decode + bf16 kernel run when flag != 0
     if (int rc = ensure_flag(h)) return rc;
-    uint32_t* flag = (uint32_t*) h->flag.p;
-    HIP_TRY(h, launch_fill_u32(flag, 0u, 1, h->stream));
-    const mme_hip_tensor* t[2] = {ta, tb};
-    const void*           base[2] = {a_base, b_base};
-    for (int i = 0; i < 2; i++)
-        if (plan.scan_kind[i] >= 0)
-            HIP_TRY(h, launch_fp8_special_scan(flag, base[i], span_elements(t[i]), t[i]->dtype == MME_HIP_FP8_143 ? 3 : 2,
-                                               plan.scan_kind[i], h->stream));
+    uint32_t*      flag = (uint32_t*) h->flag.p;
+    const uint32_t epoch = ++h->specials_epoch; // the flag holds the epoch of the latest call whose scan found something
+    HIP_TRY(h, launch_fp8_special_scan2(flag, epoch, a_base, span_elements(ta), ta->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[0], b_base,
+                                        span_elements(tb), tb->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[1], h->stream));
     g.skip_flag = flag;
-    g.skip_if = 1; // native variant: skipped when the flag is set
+    g.skip_epoch = epoch;
+    g.skip_if = 1; // native variant: skipped when the scan found something
     HIP_TRY(h, launch_gemm(g, h->stream));
 
     const size_t na = span_elements(ta), nb = span_elements(tb);
@@ -307,10 +309,9 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     HIP_TRY(h, h->decode_ws.reserve((na_pad + nb + 8) * 2));
     uint16_t* da = (uint16_t*) h->decode_ws.p;
     uint16_t* db = da + na_pad;
-    HIP_TRY(h, launch_fp8_to_bf16(da, (const uint8_t*) a_base, na, ta->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) ta->fp_bias,
-                                  ta->inf_nan_mode, flag, h->stream));
-    HIP_TRY(h, launch_fp8_to_bf16(db, (const uint8_t*) b_base, nb, tb->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) tb->fp_bias,
-                                  tb->inf_nan_mode, flag, h->stream));
+    HIP_TRY(h, launch_fp8_to_bf16_2(da, (const uint8_t*) a_base, na, ta->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) ta->fp_bias, ta->inf_nan_mode, db,
+                                    (const uint8_t*) b_base, nb, tb->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) tb->fp_bias, tb->inf_nan_mode, flag,
+                                    epoch, h->stream));
     GemmProblem g2 = g;
     g2.dtype = DT_BF16;
     g2.A.base = (const char*) da;
@@ -325,7 +326,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         g2.epi.alpha = pow2f(e);
         g2.epi.has_alpha = e != 0;
     }
-    g2.skip_if = 0; // decoded variant: skipped when the flag is clear
+    g2.skip_if = 0; // decoded variant: skipped unless the scan found something
     g2.split_k = g.split_k;
     HIP_TRY(h, launch_gemm(g2, h->stream));
     return MME_HIP_OK;

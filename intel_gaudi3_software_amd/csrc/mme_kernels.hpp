@@ -75,10 +75,12 @@ struct GemmProblem
     GemmEpilogue epi;
     int          split_k;    // >1: partial sums go to workspace and are reduced in a fixed order
     float*       workspace;  // split_k * batch * M * N floats
-    // device-side predicate: when skip_flag != NULL the whole launch returns at once if (*skip_flag != 0) == skip_if.
+    // device-side predicate: when skip_flag != NULL the whole launch returns at once if (*skip_flag == skip_epoch) == skip_if
+    // (the scan of the call with that epoch number found something; the flag is never reset, epochs only grow).
     // Lets the fp8 path enqueue "native fp8" and "decoded bf16" variants back to back without a host round trip.
     const uint32_t* skip_flag;
     int             skip_if;
+    uint32_t        skip_epoch;
 };
 
 size_t     gemm_workspace_bytes(const GemmProblem& p);
@@ -96,12 +98,16 @@ hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int 
 
 // flags every exponent-all-ones code of an fp8 buffer (inf / NaN in Gaudi's full mode, finite for the hardware's
 // e4m3): *flag |= 1.  mask_kind 0: any code with all exponent bits set; 1: only 0x7F / 0xFF.
-hipError_t launch_fp8_special_scan(uint32_t* flag, const void* data, size_t n, int man_bits, int mask_kind, hipStream_t s);
+// one launch for both operands: mask_kind < 0 leaves an operand out; a hit stores `epoch` into *flag
+hipError_t launch_fp8_special_scan2(uint32_t* flag, uint32_t epoch, const void* a, size_t na, int man_bits_a, int mask_kind_a, const void* b,
+                                    size_t nb, int man_bits_b, int mask_kind_b, hipStream_t s);
 
 // dense or strided 5-d fp8 -> bf16 exact decode (used when the hardware's fp8 formats cannot represent the operand)
 // run_flag (device, may be NULL): the kernel does nothing when *run_flag == 0
-hipError_t launch_fp8_to_bf16(uint16_t* out, const uint8_t* in, size_t n, int man_bits, int bias, int mode, const uint32_t* run_flag,
-                              hipStream_t s);
+// both operands in one launch; runs only when *run_flag == epoch (run_flag may be NULL: always)
+hipError_t launch_fp8_to_bf16_2(uint16_t* out_a, const uint8_t* in_a, size_t na, int man_bits_a, int bias_a, int mode_a, uint16_t* out_b,
+                                const uint8_t* in_b, size_t nb, int man_bits_b, int bias_b, int mode_b, const uint32_t* run_flag, uint32_t epoch,
+                                hipStream_t s);
 // one-lane fill of n 32-bit cells (kernels instead of memset nodes keep call sequences graph-capturable)
 hipError_t launch_fill_u32(uint32_t* p, uint32_t v, size_t n, hipStream_t s);
 
