@@ -607,13 +607,28 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         {
             constexpr int MAN = decltype(m_c)::value;
             walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
-                uint32_t pk[4];
+                // the hardware converter equals the reference's conversion on finite inputs; a block that holds inf or
+                // NaN (sum of magnitudes not finite) takes the exact converter
+                float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int c = 0; c < 4; c++)
+                for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
+                const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) <= 0x1.fffffep+127f);
+                uint32_t   pk[4];
+                if (__builtin_amdgcn_ballot_w64(special) == 0)
                 {
-                    pk[c] = 0;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) pk[c] |= (fp32_to_fp8_rne_mode0<MAN>(f2u(val[4 * c + e]), cp.exp_bias, cp.clip_fp, cp.clip_inf_in) & 0xFFu) << (8 * e);
+                    for (int c = 0; c < 4; c++) pk[c] = fp8_hw_pack4<MAN>(val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3], cp.exp_bias, cp.clip_fp);
+                }
+                else
+                {
+#pragma unroll
+                    for (int c = 0; c < 4; c++)
+                    {
+                        pk[c] = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            pk[c] |= (fp32_to_fp8_rne_mode0<MAN>(f2u(val[4 * c + e]), cp.exp_bias, cp.clip_fp, cp.clip_inf_in) & 0xFFu) << (8 * e);
+                    }
                 }
                 *(e_v4u*) ((uint8_t*) g.epi.out + idx) = e_v4u {pk[0], pk[1], pk[2], pk[3]};
             });

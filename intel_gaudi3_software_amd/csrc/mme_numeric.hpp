@@ -326,6 +326,34 @@ __device__ __forceinline__ uint32_t cast_elem(float v, const CastParams& p)
         return fp32_to_fp32_ref(u, p.rm, p.clip_fp, p.ftz);
 }
 
+// Four finite fp32 values -> four fp8 codes (round to nearest even, full inf/nan mode) with the hardware converter: scale
+// by 2^(bias - 7) (fp8_143) / 2^(bias - 15) (fp8_152) so that the target becomes OCP e4m3 / e5m2, clamp to the largest
+// normal (clipping) or to the first power of two beyond it (whose OCP code is this format's inf code), convert.
+// Equal to fp32_to_fp8_rne_mode0 for every finite input (checked over all 2^32 inputs for several biases, clipping on
+// and off); inf and NaN inputs must take the exact converter.
+template<int M>
+__device__ __forceinline__ uint32_t fp8_hw_pack4(float a, float b, float c, float d, int bias, int clip)
+{
+    const float scale = u2f((uint32_t) (127 + bias - (M == 3 ? 7 : 15)) << 23);
+    const float lim = M == 3 ? (clip ? 240.0f : 256.0f) : (clip ? 57344.0f : 65536.0f);
+    a = __builtin_fminf(__builtin_fmaxf(a * scale, -lim), lim);
+    b = __builtin_fminf(__builtin_fmaxf(b * scale, -lim), lim);
+    c = __builtin_fminf(__builtin_fmaxf(c * scale, -lim), lim);
+    d = __builtin_fminf(__builtin_fmaxf(d * scale, -lim), lim);
+    int r = 0;
+    if constexpr (M == 3)
+    {
+        r = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, r, false);
+        r = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, r, true);
+    }
+    else
+    {
+        r = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, r, false);
+        r = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, r, true);
+    }
+    return (uint32_t) r;
+}
+
 // whether the FAST forms apply to these parameters
 inline bool cast_params_fast(const CastParams& p)
 {
