@@ -466,6 +466,406 @@ __global__ __launch_bounds__(512) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
         (void) scaled;
     }
 }
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Resident form, for runs of output rows whose input fits in LDS at once (the benchmark shape: 14 rows of 56 pixels per
+// compute unit).  Nothing is fetched twice and nothing waits in the steady state:
+//
+//   LDS         every input row the workgroup's run needs ("virtual rows": per image segment of the run its rows plus
+//               the one above and the one below, rows outside the image as zeros), (W + 2) pixels each with zeroed
+//               halo columns, 16-byte chunks XOR-swizzled by column as above.  All of it is requested in the first
+//               microseconds, in row order, so the memory system streams the input while the first tiles are computed
+//   filter      lives in registers: a wavefront owns output channels nh * 32 .. + 31 (nh = wavefront & 1) and keeps their 36 k-step
+//               fragments (144 registers).  The filter passes through the top 72 KiB of LDS once (DMA in global order,
+//               transposing reads); input rows that overlap that area are requested after every wavefront has taken
+//               its fragments
+//   wavefront   takes pairs of pixel tiles (64 pixels of the run's flattened pixel order) from a queue in LDS, one queue
+//               per channel half, in row order: two independent accumulator chains, one ds_read_b128 per matrix-core
+//               instruction, fetched five instructions ahead; the epilogue of a pair follows its contraction
+//               immediately, which spreads the stores over the whole kernel, and the queue lets the wavefront that
+//               gets more of its SIMD's matrix-core time take more pairs
+//   sync        two workgroup barriers (filter landed, filter taken and first rows landed); the remaining rows are
+//               requested by the second wavefront of every SIMD, which waits for them and raises a counter that the
+//               others check before the first pair that needs those rows
+constexpr int CR_LDS_BYTES = 160 * 1024;
+constexpr int CR_CTRL_OFF = CR_LDS_BYTES - 16;           // three counters: the two tile queues, "all rows landed"
+constexpr int CR_STAGE_OFF = CR_CTRL_OFF - CF_WT_BYTES;  // filter staging area: the top of LDS below the counters
+constexpr int CR_MAX_TILES = 32;
+
+// number of virtual rows of a run of `rows` output rows that starts at row hs0 of an image of H rows
+__host__ __device__ inline int cr_virtual_rows(int rows, int hs0, int H)
+{
+    const int n0 = rows < H - hs0 ? rows : H - hs0;
+    const int rest = rows - n0, full = rest / H, last = rest - full * H;
+    return n0 + 2 + full * (H + 2) + (last ? last + 2 : 0);
+}
+
+// s_waitcnt vmcnt(n) for a wave-uniform n (the instruction takes an immediate); counts above 15 wait for 15
+__device__ __forceinline__ void cr_wait_vmcnt(int n)
+{
+    switch (n)
+    {
+        case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+        case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
+        case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+        case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
+        case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+        case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
+        case 6: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+        case 7: __builtin_amdgcn_s_waitcnt(0x0F77); break;
+        case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+        case 9: __builtin_amdgcn_s_waitcnt(0x0F79); break;
+        case 10: __builtin_amdgcn_s_waitcnt(0x0F7A); break;
+        case 11: __builtin_amdgcn_s_waitcnt(0x0F7B); break;
+        case 12: __builtin_amdgcn_s_waitcnt(0x0F7C); break;
+        case 13: __builtin_amdgcn_s_waitcnt(0x0F7D); break;
+        case 14: __builtin_amdgcn_s_waitcnt(0x0F7E); break;
+        default:
+            if (n < 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+            else
+                __builtin_amdgcn_s_waitcnt(0x0F7F);
+            break;
+    }
+}
+
+template<int WC> // WC: the image width when it is known at compile time (row pitch and pixel divisions become constants), else 0
+__global__ __launch_bounds__(512) void conv_fwd_resident_kernel(ConvFwdFastArgs a_by_value)
+{
+    (void) a_by_value;
+    typedef const __attribute__((address_space(4))) ConvFwdFastArgs& ArgRef;
+    ArgRef a = *(const __attribute__((address_space(4))) ConvFwdFastArgs*) __builtin_amdgcn_kernarg_segment_ptr();
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+    const int      tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int      nh = wave & 1, kg = lane >> 5;
+    const uint32_t lds_base = (uint32_t) (uintptr_t) lds;
+    uint32_t*      ctrl = (uint32_t*) (lds + CR_CTRL_OFF);
+    if (tid < 4) ctrl[tid] = 0;
+
+    // ---- filter to the staging area, first of all: its addresses need no arithmetic --------------------------------------
+    {
+        // (the workgroups that share an L2 -- every eighth -- start at different eighths of the filter, so that they do not
+        // all ask the same L2 channel for the same line at the same moment)
+        constexpr int PER_WAVE = CF_WT_BYTES / 1024 / 8;
+        const int     seg = (wave + (blockIdx.x >> 3)) & 7;
+        const char*   src = (const char*) a.w + (((lane & ~7) | ((lane & 7) ^ (((lane >> 3) & 3) << 1))) << 4) + seg * (PER_WAVE * 1024);
+#pragma unroll
+        for (int k = 0; k < PER_WAVE; k += 4)
+        {
+            const char*    g = src + k * 1024;
+            const uint32_t l = lds_base + CR_STAGE_OFF + seg * (PER_WAVE * 1024) + k * 1024;
+            if (k + 4 <= PER_WAVE)
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off\n\tglobal_load_lds_dwordx4 %0, off offset:1024\n\t"
+                             "global_load_lds_dwordx4 %0, off offset:2048\n\tglobal_load_lds_dwordx4 %0, off offset:3072" ::"v"(g), "s"(l)
+                             : "memory");
+            else
+                asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(l) : "memory");
+        }
+    }
+
+    // ---- the run and its virtual rows ------------------------------------------------------------------------------------
+    const int H = a.H, W = WC ? WC : a.W, wp = W + 2, row_bytes = wp * 128;
+    const int row_begin = blockIdx.x * a.rows_per_wg + min((int) blockIdx.x, a.rows_extra);
+    const int rows = a.rows_per_wg + ((int) blockIdx.x < a.rows_extra ? 1 : 0);
+    const int img0 = row_begin / H, hs0 = row_begin - img0 * H, n0 = min(H - hs0, rows);
+    const int V = rows <= n0 ? rows + 2 : cr_virtual_rows(rows, hs0, H);
+    const int npx = rows * W, ntiles = (npx + 31) >> 5, npairs = (ntiles + 1) >> 1;
+    // virtual row of the input row above output row o of the run
+    auto vtop = [&](int o) __attribute__((always_inline))
+    {
+        const int u = o - n0, k = cf_div(max(u, 0), H);
+        return o < n0 ? o : n0 + 2 + k * (H + 2) + (u - k * H);
+    };
+    // input row of virtual row v, counted from row 0 of image img0; -1: a row of zeros
+    auto vsrc = [&](int v) __attribute__((always_inline))
+    {
+        const int u = v - (n0 + 2), k = cf_div(max(u, 0), H + 2);
+        const int img = v < n0 + 2 ? 0 : 1 + k, h = v < n0 + 2 ? hs0 - 1 + v : u - k * (H + 2) - 1;
+        return (h >= 0 && h < H) ? img * H + h : -1;
+    };
+    // the same two for wave-uniform arguments, in scalar arithmetic
+    auto vtop_uniform = [&](int o) __attribute__((always_inline))
+    {
+        if (o < n0) return o;
+        const int u = o - n0, k = u / H;
+        return n0 + 2 + k * (H + 2) + (u - k * H);
+    };
+    auto vsrc_uniform = [&](int v) __attribute__((always_inline))
+    {
+        int img = 0, h = hs0 - 1 + v;
+        if (v >= n0 + 2)
+        {
+            const int u = v - (n0 + 2), k = u / (H + 2);
+            img = 1 + k;
+            h = u - k * (H + 2) - 1;
+        }
+        return (h >= 0 && h < H) ? img * H + h : -1;
+    };
+    const char* xbase = (const char*) (a.x + (long long) img0 * H * W * CF_C);
+    // Requests for virtual rows [va, vb): a request moves 8 consecutive pixels of one input row (64 lanes x 16 bytes) to
+    // their 8 slots of the LDS row; chunk i of the slot of LDS column c holds input channels 8 * (i ^ ((c >> 1) & 7)) .. + 7.
+    // Request k of a row starts at input column 8 k = LDS column 8 k + 1, so the lane's source offset inside the request is
+    // one of two constants (k even / odd), and the instruction's offset field steps through the row in the global and the
+    // LDS address alike: a row costs a few scalar instructions.  Whole rows are dealt to the wavefronts in turn; rows of zeros are not requested (zero_rows writes them).  Returns this wavefront's number of requests
+    const int      kw = (W + 7) >> 3;
+    const int      dj = lane >> 3, di = lane & 7;
+    const uint32_t src_even = (uint32_t) (dj * 128 + ((di ^ (((1 + dj) >> 1) & 7)) << 4));
+    const uint32_t src_odd = (uint32_t) (dj * 128 + ((di ^ ((4 + ((1 + dj) >> 1)) & 7)) << 4));
+    auto issue_rows = [&](int va, int vb, int w0, int nw) __attribute__((always_inline)) // rows to wavefronts w0 .. w0 + nw - 1
+    {
+        int n = 0;
+        if (wave < w0) return n;
+        for (int v = va + ((wave - w0 - va) & (nw - 1)); v < vb; v += nw)
+        {
+            const int g = vsrc_uniform(v);
+            if (g < 0) continue;
+            // (the values are wave-uniform; readfirstlane tells the compiler so where it cannot prove it)
+            const uint64_t src = (uint64_t) (xbase + (long long) g * W * (CF_C * 2));
+            uint64_t       src_s = (uint64_t) (uint32_t) __builtin_amdgcn_readfirstlane((uint32_t) src) |
+                             ((uint64_t) (uint32_t) __builtin_amdgcn_readfirstlane((uint32_t) (src >> 32)) << 32);
+            uint32_t dst = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t) ((v * wp + 1) * 128));
+            int      k = 0;
+            for (; k + 4 <= (W >> 3); k += 4, src_s += 4096, dst += 4096)
+                asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024\n\t"
+                             "global_load_lds_dwordx4 %0, %2 offset:2048\n\tglobal_load_lds_dwordx4 %1, %2 offset:3072" ::"v"(src_even),
+                             "v"(src_odd), "s"(src_s), "s"(dst)
+                             : "memory");
+            for (; k < kw; k++, src_s += 1024, dst += 1024)
+                if (8 * k + dj < W) cf_dma16_off((const void*) src_s, (k & 1) ? src_odd : src_even, dst);
+            n += kw;
+        }
+        return n;
+    };
+    auto zero_cols = [&](int va, int vb, int t0, int nthreads) __attribute__((always_inline))
+    {
+        for (int i = tid - t0; i < (vb - va) * 16; i += nthreads)
+        {
+            const int row = va + (i >> 4), side = (i >> 3) & 1, chunk = i & 7;
+            *reinterpret_cast<uint4*>(lds + ((row * wp + (side ? W + 1 : 0)) * 8 + chunk) * 16) = make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto zero_rows = [&](int va, int vb, int t0, int nthreads) __attribute__((always_inline))
+    {
+        auto zero_row = [&](int v) __attribute__((always_inline))
+        {
+            for (int c = tid - t0; c < wp * 8; c += nthreads) *reinterpret_cast<uint4*>(lds + (v * wp * 8 + c) * 16) = make_uint4(0, 0, 0, 0);
+        };
+        if (rows <= n0)
+        {
+            // one image segment: only its first and last virtual row can lie outside the image
+            if (hs0 == 0 && va <= 0 && 0 < vb) zero_row(0);
+            if (hs0 + n0 == H && va <= n0 + 1 && n0 + 1 < vb) zero_row(n0 + 1);
+        }
+        else
+            for (int v = va; v < vb; v++)
+                if (vsrc_uniform(v) < 0) zero_row(v);
+    };
+    // two groups of rows: [0, g0) is what tiles 0 .. 7 read (as far as it lies below the staging area), requested now;
+    // the rest follows when the staging area is free
+    const int g1 = min(V, CR_STAGE_OFF / row_bytes);
+    const int g0 = min(g1, vtop_uniform((min(npx, 256) - 1) / W) + 3);
+    const int n_g0 = issue_rows(0, g0, 0, 8);
+    zero_cols(0, g1, 0, 512);
+    zero_rows(0, g1, 0, 512);
+
+    const bool       fused = a.epi.fused != 0;
+    const bool       has_alpha = a.epi.has_alpha != 0;
+    const float      alpha = a.epi.alpha;
+    const int32_t*   col_exp = a.epi.col_exp;
+    const int        dt = fused ? a.epi.out_dtype : DT_FP32;
+    const bool       bf16_fast = fused && dt == DT_BF16 && a.epi.fast_cast;
+    const CastParams cp = {a.epi.cast.dtype,       a.epi.cast.exp_bias, a.epi.cast.inf_nan_mode, a.epi.cast.rm,    a.epi.cast.clip_fp,
+                           a.epi.cast.clip_inf_in, a.epi.cast.ftz,      a.epi.cast.relu,         a.epi.cast.scale, a.epi.cast.has_scale};
+
+    cr_wait_vmcnt(n_g0); // requests retire in issue order: the filter came first
+    __syncthreads();     // every wavefront's part of the filter has landed
+
+    // ---- this wavefront's half of the filter into registers: fragment of k-step (tap, 16 in channels) = out channel
+    // nh * 32 + lane % 32, in channels 8 * kg .. + 7 of the step; two ds_read_b64_tr_b16 as in the kernel above ---------------
+    CfFrag fw[CF_TAPS * 4];
+    {
+        const int   g = lane >> 4, j = lane & 15;
+        const char* p0 = lds + CR_STAGE_OFF + ((g >> 1) * 8 + (j >> 2)) * 128 + (((nh * 2 + (g & 1)) ^ (j >> 2)) << 5) + ((j & 3) << 3);
+#pragma unroll
+        for (int step = 0; step < CF_TAPS * 4; step++)
+        {
+            const char* p = p0 + (step >> 2) * 8192 + (step & 3) * 2048;
+            fw[step].h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((CF_LDS cf_v4s*) p);
+            fw[step].h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((CF_LDS cf_v4s*) (p + 512));
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70); // this wavefront's requests for the first group of rows
+    __syncthreads(); // everybody has taken its fragments: the staging area becomes input rows; the first rows have landed
+    // The remaining rows, by the second wavefront of each SIMD: the first one has priority on the matrix cores and starts
+    // on the pairs that read only the first rows meanwhile.  The four raise the counter when their requests have landed
+    if (wave >= 4)
+    {
+        issue_rows(g0, V, 4, 4);
+        zero_cols(g1, V, 256, 256);
+        zero_rows(g1, V, 256, 256);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (lane == 0) __hip_atomic_fetch_add(ctrl + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+
+    bool landed = false; // this wavefront has seen the counter at 4
+    while (true)
+    {
+        uint32_t q = 0;
+        if (lane == 0) q = __hip_atomic_fetch_add(ctrl + nh, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        q = __builtin_amdgcn_readfirstlane(q);
+        if ((int) q >= npairs) break;
+        const int tile0 = 2 * (int) q;
+        const int nt = tile0 + 1 < ntiles ? 2 : 1;
+        if (!landed && vtop_uniform((min(npx, (tile0 + 2) * 32) - 1) / W) + 3 > g0)
+        {
+            // every wavefront that raises the counter does so without waiting for anybody: the spin ends
+            while (__hip_atomic_load(ctrl + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < 4u) __builtin_amdgcn_s_sleep(1);
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            landed = true;
+        }
+
+        // LDS address of this lane's pixel under tap (r, s), k-step quarter 0; quarter ks is that ^ (ks << 5).  With a
+        // compile-time width the row pitch goes into the instruction's offset field and only r = 0 is kept
+        constexpr int XR = WC ? 1 : 3;
+        uint32_t      xa[2][XR][3];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+        {
+            const int p = min((tile0 + t) * 32 + (lane & 31), npx - 1);
+            const int o = cf_div(p, W), col = p - o * W, vt = vtop(o);
+#pragma unroll
+            for (int r = 0; r < XR; r++)
+#pragma unroll
+                for (int s = 0; s < 3; s++)
+                    xa[t][r][s] = (uint32_t) (((vt + r) * wp + col + s) * 128) | (uint32_t) ((kg ^ (((col + s) >> 1) & 7)) << 4);
+        }
+        v16f acc[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[t][v] = 0.0f;
+
+        // 36 k-steps x NT tiles = one flat sequence of (pixel fragment read, matrix-core instruction) pairs; the read runs
+        // DEPTH pairs ahead of its use through a ring of DEPTH + 1 fragments, which is what hides the LDS latency: a
+        // wavefront issues nothing while its own matrix-core instruction runs, so every wait it meets is exposed
+        auto contract = [&](auto nt_c) __attribute__((always_inline))
+        {
+            constexpr int NT = decltype(nt_c)::value;
+            constexpr int NQ = CF_TAPS * 4 * NT, DEPTH = WC ? 5 : 2, RING = DEPTH + 1;
+            CfFrag        fx[RING];
+            auto ld_x = [&](int q) __attribute__((always_inline))
+            {
+                const int step = q / NT, t = q - step * NT, tap = step >> 2, ks = step & 3, r = tap / 3, s = tap - r * 3;
+                if constexpr (WC != 0)
+                    fx[q % RING].u = *reinterpret_cast<const uint4*>(lds + (xa[t][0][s] ^ (uint32_t) (ks << 5)) + r * ((WC + 2) * 128));
+                else
+                    fx[q % RING].u = *reinterpret_cast<const uint4*>(lds + (xa[t][r][s] ^ (uint32_t) (ks << 5)));
+            };
+#pragma unroll
+            for (int q = 0; q < DEPTH; q++) ld_x(q);
+#pragma unroll
+            for (int q = 0; q < NQ; q++)
+            {
+                const int step = q / NT, t = q - step * NT;
+                if (q + DEPTH < NQ) ld_x(q + DEPTH);
+                __builtin_amdgcn_sched_barrier(0);
+                acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[step].v, fx[q % RING].v, acc[t], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        if (nt == 2) contract(std::integral_constant<int, 2>());
+        else
+            contract(std::integral_constant<int, 1>());
+
+        // ---- epilogue of the pair: accumulator register v of lane l = channel nh * 32 + 8 * (v / 4) + 4 * (l / 32) + v % 4
+        // of pixel l % 32; v_permlane32_swap leaves the lane with channels nh * 32 + kg * 16 + 0 .. 15 in order -------------
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+        {
+            if (t == 1 && nt < 2) break;
+            const int p = (tile0 + t) * 32 + (lane & 31);
+            float val[16];
+#pragma unroll
+            for (int g = 0; g < 2; g++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                {
+                    const float lo = acc[t][4 * g + i], hi = acc[t][8 + 4 * g + i];
+                    const auto  sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                    val[8 * g + i] = __uint_as_float(sw[0]);
+                    val[8 * g + 4 + i] = __uint_as_float(sw[1]);
+                }
+            if (has_alpha)
+            {
+#pragma unroll
+                for (int c = 0; c < 16; c++) val[c] *= alpha;
+            }
+            if (col_exp)
+            {
+#pragma unroll
+                for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[nh * 32 + kg * 16 + c]);
+            }
+            const long long idx = ((long long) row_begin * W + p) * CF_K + nh * 32 + kg * 16;
+            if (bf16_fast)
+            {
+                // v_cvt_pk_bf16_f32 where it gives the reference's code (everything but NaN, and inf / overflow where
+                // clipping matters); the sum of |x| over the lane's 16 values detects the rest
+                uint32_t pk[8];
+                auto     convert = [&](auto relu_c) __attribute__((always_inline))
+                {
+                    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int c = 0; c < 16; c++)
+                    {
+                        if (decltype(relu_c)::value) val[c] = relu_ref(val[c]);
+                        sum[c & 3] += __builtin_fabsf(val[c]);
+                    }
+                    const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
+                    if (__builtin_amdgcn_ballot_w64(special) == 0)
+                    {
+#pragma unroll
+                        for (int c = 0; c < 8; c++)
+                        {
+                            const cf_v2bf h = __builtin_convertvector(cf_v2f {val[2 * c], val[2 * c + 1]}, cf_v2bf);
+                            __builtin_memcpy(&pk[c], &h, 4);
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for (int c = 0; c < 8; c++)
+                            pk[c] = fp32_to_bf16_rne(f2u(val[2 * c]), cp.clip_fp, cp.clip_inf_in) |
+                                    (fp32_to_bf16_rne(f2u(val[2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
+                    }
+                };
+                if (cp.relu) convert(std::true_type());
+                else
+                    convert(std::false_type());
+                if (p < npx)
+                {
+                    cf_v4u* o = (cf_v4u*) ((uint16_t*) a.epi.out + idx);
+                    o[0] = cf_v4u {pk[0], pk[1], pk[2], pk[3]};
+                    o[1] = cf_v4u {pk[4], pk[5], pk[6], pk[7]};
+                }
+            }
+            else if (p < npx)
+            {
+                if (!fused)
+                {
+                    cf_v4f* o = (cf_v4f*) ((float*) a.epi.out + idx);
+#pragma unroll
+                    for (int c = 0; c < 4; c++) o[c] = cf_v4f {val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3]};
+                }
+                else
+                {
+#pragma unroll 1
+                    for (int c = 0; c < 16; c++) store_out_slow(a.epi, idx + c, val[c]);
+                }
+            }
+        }
+    }
+}
 } // namespace
 
 bool conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int W, int H, int D, const int stride[4], const int dil[4],
@@ -502,6 +902,36 @@ hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int 
     const int grid = (int) std::min<long long>((rows + CF_TR - 1) / CF_TR, num_cus > 0 ? num_cus : 256);
     a.rows_per_wg = (int) (rows / grid);
     a.rows_extra = (int) (rows % grid);
+    // the resident form needs every workgroup's input rows in LDS at once and at most four rounds of tiles
+    bool resident = (long long) (a.rows_per_wg + 1) * W <= CR_MAX_TILES * 32;
+    for (int wg = 0; wg < grid && resident; wg++)
+    {
+        const long long row_begin = (long long) wg * a.rows_per_wg + std::min(wg, a.rows_extra);
+        const int       n = a.rows_per_wg + (wg < a.rows_extra ? 1 : 0);
+        if (n * W > CR_MAX_TILES * 32 || cr_virtual_rows(n, (int) (row_begin % H), H) * (W + 2) * 128 > CR_CTRL_OFF) resident = false;
+    }
+    if (resident)
+    {
+        static bool attr2_done = false;
+        if (!attr2_done)
+        {
+            for (const void* f : {(const void*) conv_fwd_resident_kernel<0>, (const void*) conv_fwd_resident_kernel<56>,
+                                  (const void*) conv_fwd_resident_kernel<28>, (const void*) conv_fwd_resident_kernel<14>})
+            {
+                hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_BYTES);
+                if (e != hipSuccess) return e;
+            }
+            attr2_done = true;
+        }
+        if (W == 56) hipLaunchKernelGGL(conv_fwd_resident_kernel<56>, dim3(grid), dim3(512), CR_LDS_BYTES, s, a);
+        else if (W == 28)
+            hipLaunchKernelGGL(conv_fwd_resident_kernel<28>, dim3(grid), dim3(512), CR_LDS_BYTES, s, a);
+        else if (W == 14)
+            hipLaunchKernelGGL(conv_fwd_resident_kernel<14>, dim3(grid), dim3(512), CR_LDS_BYTES, s, a);
+        else
+            hipLaunchKernelGGL(conv_fwd_resident_kernel<0>, dim3(grid), dim3(512), CR_LDS_BYTES, s, a);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(conv_fwd_fast_kernel, dim3(grid), dim3(512), lds_bytes, s, a);
     return hipGetLastError();
 }
