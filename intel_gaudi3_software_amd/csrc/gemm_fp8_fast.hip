@@ -825,16 +825,18 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
     const int       nk = p.K * (p.dtype == DT_BF16 ? 2 : 1) / FBK;
     int             best = 1;
     // Splitting the reduction pays when the tiles leave most of the chip idle and the reduction is long: a slice costs a
-    // pass of the fp32 output through the workspace plus the reduction kernel.  Rough model in microseconds: a stage
-    // takes 0.5, the workspace moves at 4 TB/s, the extra launch costs 6.  Every slice keeps an even number of stages,
-    // at least 6.
+    // pass of the fp32 output through the workspace plus the reduction kernel.  Rough model in microseconds: a stage (128 bytes of
+    // k per row) takes 1.0 as measured on full-size fp8 and bf16 problems, the workspace moves at 3 TB/s (the reduction
+    // kernel's measured rate is 2.3 .. 3.1), the extra launch costs 6.  Every slice keeps an even number of stages, at least 6.
+    const double stage_us = 1.0;
     const double out_bytes = 8.0 * p.M * (double) p.N * p.batch[0] * p.batch[1] * p.batch[2];
-    double       best_t = (double) ((tiles + num_cus - 1) / num_cus) * nk * 0.5;
+    const double t1 = (double) ((tiles + num_cus - 1) / num_cus) * nk * stage_us;
+    double       best_t = 0.8 * t1; // a split has to promise a clear gain
     for (int s = 2; s <= 64; s++)
     {
         if (nk % (2 * s) || nk / s < 6) continue;
-        const double t = (double) ((tiles * s + num_cus - 1) / num_cus) * (nk / s) * 0.5 + s * out_bytes / 4e6 + 6.0;
-        if (t < 0.8 * best_t)
+        const double t = (double) ((tiles * s + num_cus - 1) / num_cus) * (nk / s) * stage_us + s * out_bytes / 3e6 + 6.0;
+        if (t < best_t)
         {
             best_t = t;
             best = s;
