@@ -12,6 +12,15 @@ hipError_t launch_cast_from_fp32(void* out, const float* in, size_t n, const Cas
                                  size_t n_cols, hipStream_t s);
 hipError_t launch_cast_to_fp32(float* out, const void* in, int dtype, int bias, int mode, size_t n, float scale,
                                int has_scale, const int32_t* col_exp, size_t n_cols, hipStream_t s);
+// stochastic rounding / stochastic flush: regs = the calculator's LFSR registers 0 .. 127 before the call, jump = device table of
+// LFSR_JUMP_LEVELS x 32 words (image of every state bit under 2^k steps); reseed: step a register after every use
+constexpr int LFSR_JUMP_LEVELS = 40;
+struct LfsrRegisters
+{
+    uint32_t v[128];
+};
+hipError_t launch_cast_stochastic(void* out, const float* in, size_t n, const CastParams& p, int sftz, int reseed, uint32_t polynomial,
+                                  const LfsrRegisters& regs, const uint32_t* jump, hipStream_t s);
 hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s);
 hipError_t launch_absmax(float* out, const float* in, size_t n, hipStream_t s);
 
