@@ -486,6 +486,36 @@ hipError_t launch_cast_stochastic(void* out, const float* in, size_t n, const Ca
     return hipGetLastError();
 }
 
+// ---- weights of transposed_dedx: out[i0][i1][s][r][q] = in[i1][i0][S - 1 - s][r][q] (first index contiguous on both
+// sides), i.e. transposeTensor + reverseWeightsDimS of the reference (mme_reference_impl.cpp:324-393, 625-647) -----------
+template<typename T>
+__global__ __launch_bounds__(CAST_THREADS) void repack_transposed_weights_kernel(T* __restrict__ out, const T* __restrict__ in, uint32_t n0, uint32_t n1,
+                                                                                 uint32_t S, size_t total)
+{
+    const size_t stride = (size_t) gridDim.x * CAST_THREADS;
+    for (size_t i = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x; i < total; i += stride)
+    {
+        // i = i0 + n1 * (i1 + n0 * (s + S * rq))
+        const size_t   a = i / n1, b = a / n0, rq = b / S;
+        const uint32_t i0 = (uint32_t) (i - a * n1), i1 = (uint32_t) (a - b * n0), s = (uint32_t) (b - rq * S);
+        out[i] = in[i1 + (size_t) n0 * (i0 + (size_t) n1 * ((S - 1 - s) + (size_t) S * rq))];
+    }
+}
+
+hipError_t launch_repack_transposed_weights(void* out, const void* in, int elem_size, uint32_t n0, uint32_t n1, uint32_t S, size_t total, hipStream_t s)
+{
+    if (total == 0) return hipSuccess;
+    const dim3 grid(grid_for(total, 4096)), block(CAST_THREADS);
+    switch (elem_size)
+    {
+        case 1: hipLaunchKernelGGL(repack_transposed_weights_kernel<uint8_t>, grid, block, 0, s, (uint8_t*) out, (const uint8_t*) in, n0, n1, S, total); break;
+        case 2: hipLaunchKernelGGL(repack_transposed_weights_kernel<uint16_t>, grid, block, 0, s, (uint16_t*) out, (const uint16_t*) in, n0, n1, S, total); break;
+        case 4: hipLaunchKernelGGL(repack_transposed_weights_kernel<uint32_t>, grid, block, 0, s, (uint32_t*) out, (const uint32_t*) in, n0, n1, S, total); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s)
 {
     if (n == 0) return hipSuccess;

@@ -53,6 +53,7 @@ struct mme_hip_calc
     uint32_t              polynomial = 0;
     std::vector<uint32_t> lfsr_jump;       // LFSR_JUMP_LEVELS x 32 words, built on first use
     DeviceBuffer          lfsr_jump_dev;
+    DeviceBuffer          weights_ws;      // repacked weights of transposed_dedx
     std::string           error;
     DeviceBuffer          split_ws;  // split-k partial sums
     DeviceBuffer          decode_ws; // bf16 copies of fp8 operands the hardware formats cannot express
@@ -525,8 +526,33 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
 {
     if (!h) return MME_HIP_EINVAL;
     if (!cp) return fail(h, MME_HIP_EINVAL, "got null pointer");
-    if (op == MME_HIP_OP_TRANSPOSED_DEDX || op == MME_HIP_OP_DETERMINISTIC_DEDW)
-        return fail(h, MME_HIP_EUNSUPPORTED, "op %d is not built in this library", op);
+    if (op == MME_HIP_OP_DETERMINISTIC_DEDW) return fail(h, MME_HIP_EUNSUPPORTED, "op %d is not built in this library", op);
+    if (op == MME_HIP_OP_TRANSPOSED_DEDX)
+    {
+        // mme_reference_impl.cpp:625-647: exchange the first two weight dimensions, reverse the S axis, then dedx.  The
+        // weights are small; they are repacked into a workspace by one launch, as the reference does on the host
+        if (int rc = check_tensor(h, w, "inputB")) return rc;
+        uint64_t acc = 1;
+        for (int d = 0; d < 5; d++)
+        {
+            if (w->sizes[d] > 1 && w->strides[d] != acc) return fail(h, MME_HIP_EUNSUPPORTED, "strided weight tensors are not built in this library");
+            acc *= w->sizes[d];
+        }
+        const int es = elem_size(w->dtype);
+        HIP_TRY(h, h->weights_ws.reserve((size_t) acc * es + 16));
+        HIP_TRY(h, launch_repack_transposed_weights(h->weights_ws.p, w->data, es, w->sizes[0], w->sizes[1], w->sizes[2], (size_t) acc, h->stream));
+        mme_hip_tensor wr = *w;
+        wr.data = h->weights_ws.p;
+        wr.sizes[0] = w->sizes[1];
+        wr.sizes[1] = w->sizes[0];
+        acc = 1;
+        for (int d = 0; d < 5; d++)
+        {
+            wr.strides[d] = (uint32_t) acc;
+            acc *= wr.sizes[d];
+        }
+        return mme_hip_convolution_dev(h, out, x, &wr, y, cp, MME_HIP_OP_DEDX, epi);
+    }
     if (op != MME_HIP_OP_FWD && op != MME_HIP_OP_DEDX && op != MME_HIP_OP_DEDW) return fail(h, MME_HIP_EINVAL, "invalid operation");
     // operand roles (mme_reference_impl.cpp:611-655): fwd A=x B=w; dedx A=y B=w; dedw A=x B=y
     const mme_hip_tensor* A = op == MME_HIP_OP_DEDX ? y : x;

@@ -21,6 +21,9 @@ struct LfsrRegisters
 };
 hipError_t launch_cast_stochastic(void* out, const float* in, size_t n, const CastParams& p, int sftz, int reseed, uint32_t polynomial,
                                   const LfsrRegisters& regs, const uint32_t* jump, hipStream_t s);
+// weights of transposed_dedx (dense, n0 x n1 x S x R x Q, n0 contiguous) -> n1 x n0 x S x R x Q with the S axis reversed
+hipError_t launch_repack_transposed_weights(void* out, const void* in, int elem_size, uint32_t n0, uint32_t n1, uint32_t S, size_t total,
+                                            hipStream_t s);
 hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s);
 hipError_t launch_absmax(float* out, const float* in, size_t n, hipStream_t s);
 

@@ -750,6 +750,39 @@ static char* densify(const mme_hip_tensor* t)
 int orc_convolution(const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w,
                     const mme_hip_tensor* y, const mme_hip_conv_params* p, int op, int rm)
 {
+    if (op == MME_HIP_OP_TRANSPOSED_DEDX)
+    {
+        /* mme_reference_impl.cpp:625-647: the weights arrive with their first two dimensions exchanged (transposeTensor,
+         * :366-393) and are read with the S axis reversed (reverseWeightsDimS, :324-364); then a plain dedx */
+        if (!w || !w->data) return fail("got null pointer");
+        const int       wes = dtype_size(w->dtype);
+        const uint64_t  n0 = w->sizes[0], n1 = w->sizes[1], S = w->sizes[2], R = w->sizes[3], Q = w->sizes[4];
+        char*           buf = (char*) malloc((size_t) (n0 * n1 * S * R * Q ? n0 * n1 * S * R * Q : 1) * wes);
+        mme_hip_tensor  wr = *w;
+        uint64_t        acc = 1;
+        wr.sizes[0] = (uint32_t) n1;
+        wr.sizes[1] = (uint32_t) n0;
+        for (int d = 0; d < 5; d++)
+        {
+            wr.strides[d] = (uint32_t) acc;
+            acc *= wr.sizes[d];
+        }
+        wr.data = buf;
+        for (uint64_t q = 0; q < Q; q++)
+            for (uint64_t r = 0; r < R; r++)
+                for (uint64_t sx = 0; sx < S; sx++)
+                    for (uint64_t i1 = 0; i1 < n0; i1++)
+                        for (uint64_t i0 = 0; i0 < n1; i0++)
+                        {
+                            const uint64_t src = i1 * w->strides[0] + i0 * w->strides[1] + (S - 1 - sx) * w->strides[2] + r * w->strides[3] +
+                                                 q * w->strides[4];
+                            const uint64_t dst = i0 + n1 * (i1 + n0 * (sx + S * (r + R * q)));
+                            memcpy(buf + dst * wes, (const char*) w->data + src * wes, (size_t) wes);
+                        }
+        const int rc = orc_convolution(out, x, &wr, y, p, MME_HIP_OP_DEDX, rm);
+        free(buf);
+        return rc;
+    }
     const mme_hip_tensor *A, *B;
     switch (op)
     {
