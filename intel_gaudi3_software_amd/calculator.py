@@ -201,12 +201,9 @@ class HipCalculator:
                        int(stochasticFTZfp8)))
 
     def doMemoryWrite(self, memory, mmeOut, reductionOp=abi.REDUCTION_NONE, reductionRm=0, clipFp=False):
-        if memory.is_device or mmeOut.is_device:
-            if reductionOp != abi.REDUCTION_NONE:
-                raise MMEStackException("memory-write reductions are not built in this library", abi.EUNSUPPORTED)
-            memory.data().view(-1)[:] = mmeOut.data().view(-1)[:memory.data().numel()]
-            return
-        self._check(self._lib.mme_hip_memory_write(self._h, memory.desc, mmeOut.desc, reductionOp, reductionRm, int(clipFp)))
+        dev = self._placement(memory, mmeOut)
+        fn = self._lib.mme_hip_memory_write_dev if dev else self._lib.mme_hip_memory_write
+        self._check(fn(self._h, memory.desc, mmeOut.desc, reductionOp, reductionRm, int(clipFp)))
 
     # ---- extensions of the GPU path ------------------------------------------------------------------------------------
     def synchronize(self):

@@ -900,18 +900,62 @@ int mme_hip_activation(mme_hip_handle h, const mme_hip_tensor* out, const mme_hi
     return MME_HIP_OK;
 }
 
+int mme_hip_memory_write_dev(mme_hip_handle h, const mme_hip_tensor* memory, const mme_hip_tensor* mme_out, int reduction_op, int reduction_rm,
+                             int clip_fp)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (!memory || !mme_out) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    if (reduction_op < 0 || reduction_op > MME_HIP_REDUCTION_NONE) return fail(h, MME_HIP_EINVAL, "invalid reduction operation %d", reduction_op);
+    const size_t n = (size_t) span_elements(memory);
+    if (n && (!memory->data || !mme_out->data)) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    if (reduction_op == MME_HIP_REDUCTION_NONE)
+    {
+        // a byte copy of the destination tensor's size (mme_reference_impl.cpp:725-729)
+        const size_t bytes = n * elem_size(memory->dtype);
+        if (bytes) HIP_TRY(h, hipMemcpyAsync(memory->data, mme_out->data, bytes, hipMemcpyDeviceToDevice, h->stream));
+        return MME_HIP_OK;
+    }
+    // element types of a reduction: convertDataTypeToDataTypeRMW, mme_reference_impl.cpp:691-716
+    switch (memory->dtype)
+    {
+        case MME_HIP_BF16:
+        case MME_HIP_FP32: break;
+        case MME_HIP_FP8_143: return fail(h, MME_HIP_EINVAL, "fp8_143 is not supported in reduction");
+        case MME_HIP_FP8_152:
+        case MME_HIP_FP16: return fail(h, MME_HIP_EUNSUPPORTED, "fp8_152 / fp16 reductions are not built in this library");
+        default: return fail(h, MME_HIP_EINVAL, "Unsupported data type when converting to reduction RMW data type");
+    }
+    if (mme_out->dtype != memory->dtype) return fail(h, MME_HIP_EINVAL, "element types of memory and mmeOut differ");
+    if (reduction_rm < 0 || reduction_rm > 3) return fail(h, MME_HIP_EINVAL, "invalid reduction rounding mode %d", reduction_rm);
+    HIP_TRY(h, launch_memory_write_reduce(memory->data, mme_out->data, memory->dtype == MME_HIP_FP32 ? DT_FP32 : DT_BF16, n, reduction_op, reduction_rm,
+                                          clip_fp, h->stream));
+    return MME_HIP_OK;
+}
+
 int mme_hip_memory_write(mme_hip_handle h, const mme_hip_tensor* memory, const mme_hip_tensor* mme_out, int reduction_op, int reduction_rm,
                          int clip_fp)
 {
-    (void) reduction_rm;
-    (void) clip_fp;
     if (!h) return MME_HIP_EINVAL;
     if (!memory || !mme_out) return fail(h, MME_HIP_EINVAL, "got null pointer");
-    if (reduction_op != MME_HIP_REDUCTION_NONE) return fail(h, MME_HIP_EUNSUPPORTED, "memory-write reductions are not built in this library");
-    // reduction none: a byte copy of the destination tensor's size (mme_reference_impl.cpp:725-729)
-    const size_t bytes = (size_t) span_elements(memory) * elem_size(memory->dtype);
-    if (bytes) memmove(memory->data, mme_out->data, bytes);
-    return MME_HIP_OK;
+    if (reduction_op == MME_HIP_REDUCTION_NONE)
+    {
+        // reduction none: a byte copy of the destination tensor's size (mme_reference_impl.cpp:725-729), host to host
+        const size_t bytes = (size_t) span_elements(memory) * elem_size(memory->dtype);
+        if (bytes) memmove(memory->data, mme_out->data, bytes);
+        return MME_HIP_OK;
+    }
+    // the reduction reads memory's span of elements from both buffers
+    mme_hip_tensor o = *mme_out;
+    for (int d = 0; d < 5; d++)
+    {
+        o.sizes[d] = memory->sizes[d];
+        o.strides[d] = memory->strides[d];
+    }
+    Staged sm, so;
+    if (int rc = stage_in(h, sm, memory, true)) return rc;
+    if (int rc = stage_in(h, so, &o, true)) return rc;
+    if (int rc = mme_hip_memory_write_dev(h, &sm.t, &so.t, reduction_op, reduction_rm, clip_fp)) return rc;
+    return stage_out(h, sm);
 }
 
 } // extern "C"

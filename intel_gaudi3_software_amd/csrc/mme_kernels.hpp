@@ -24,6 +24,9 @@ hipError_t launch_cast_stochastic(void* out, const float* in, size_t n, const Ca
 // weights of transposed_dedx (dense, n0 x n1 x S x R x Q, n0 contiguous) -> n1 x n0 x S x R x Q with the S axis reversed
 hipError_t launch_repack_transposed_weights(void* out, const void* in, int elem_size, uint32_t n0, uint32_t n1, uint32_t S, size_t total,
                                             hipStream_t s);
+// memory[i] = memory[i] (op) mme_out[i] for fp32 / bf16 (op: 0 add, 1 sub, 2 min, 3 max, 4 max(sum, 0); rm: 0 nearest even, 1 toward
+// zero, 2 up, 3 down)
+hipError_t launch_memory_write_reduce(void* memory, const void* mme_out, int dtype, size_t n, int op, int rm, int clip, hipStream_t s);
 hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s);
 hipError_t launch_absmax(float* out, const float* in, size_t n, hipStream_t s);
 

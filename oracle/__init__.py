@@ -12,6 +12,7 @@ import subprocess
 _HERE = os.path.dirname(os.path.abspath(__file__))
 ORACLE_SO = os.path.join(_HERE, "libmme_oracle.so")
 REF_SO = os.path.join(_HERE, "_ref", "libmme_ref.so")
+REF_RMW_SO = os.path.join(_HERE, "_ref", "libmme_ref_rmw.so")
 
 u8p, u16p, u32p, i32p, f32p = (C.POINTER(t) for t in (C.c_uint8, C.c_uint16, C.c_uint32, C.c_int32, C.c_float))
 vp = C.c_void_p
@@ -70,6 +71,7 @@ def oracle():
         L.orc_fp32_to_fp32_n.argtypes = [vp, vp, C.c_size_t] + [C.c_int] * 4
         L.orc_add_fp32_n.argtypes = [vp, vp, vp, C.c_size_t, C.c_int]
         L.orc_tree9_n.argtypes = [vp, vp, vp, C.c_size_t, C.c_int]
+        L.orc_memory_write.argtypes = [vp, vp, C.c_int, C.c_int, C.c_int]
         _oracle = L
     return _oracle
 
@@ -98,3 +100,19 @@ def ref():
         L.ref_fma_vec.argtypes = [vp, vp, C.c_uint, C.c_int, C.c_int, C.c_uint, C.c_uint, C.c_int, C.c_int]
         _ref = L
     return _ref
+
+
+_ref_rmw = None
+
+
+def ref_rmw():
+    """The reference's memory-write reduction (executeOp), compiled at -O0 (see the Makefile), or None when not built."""
+    global _ref_rmw
+    if _ref_rmw is None:
+        if not os.path.exists(REF_RMW_SO):
+            return None
+        L = C.CDLL(REF_RMW_SO)
+        L.ref_memory_write_words.argtypes = [vp, vp, C.c_size_t] + [C.c_int] * 4
+        L.ref_memory_write_words.restype = None
+        _ref_rmw = L
+    return _ref_rmw

@@ -129,6 +129,39 @@ static void reference_gemm_simple_test_fp8(Calculator& calculator)
     }
 }
 
+// doMemoryWrite with a reduction, through shared pointers like the reference's callers (mme_reference.h:174-178): values
+// chosen so that the result is known in closed form
+static void memory_write_reductions(Calculator& calculator)
+{
+    // fp32 add, nearest even: 1 + 2^-24 is a tie and stays 1; round up makes it the next float; max_0 clamps a negative sum
+    std::vector<float> mem = {1.0f, 1.0f, -3.0f, 2.5f}, out = {5.9604645e-08f, 5.9604645e-08f, 1.0f, -1.0f};
+    auto               m = std::make_shared<Tensor>(SizeArray {4, 1, 1, 1, 1}, 1, MME_HIP_FP32, mem.data());
+    auto               o = std::make_shared<Tensor>(SizeArray {4, 1, 1, 1, 1}, 1, MME_HIP_FP32, out.data());
+    calculator.doMemoryWrite(m, o, MME_HIP_REDUCTION_ADD, MME_HIP_REDUCTION_RM_NEAREST_EVEN);
+    EXPECT(mem[0] == 1.0f && mem[2] == -2.0f && mem[3] == 1.5f);
+    mem = {1.0f, 1.0f, -3.0f, 2.5f};
+    calculator.doMemoryWrite(m, o, MME_HIP_REDUCTION_ADD, MME_HIP_REDUCTION_RM_UP);
+    EXPECT(mem[0] == std::nextafter(1.0f, 2.0f) && mem[2] == -2.0f);
+    mem = {1.0f, 1.0f, -3.0f, 2.5f};
+    calculator.doMemoryWrite(m, o, MME_HIP_REDUCTION_MAX_0, MME_HIP_REDUCTION_RM_NEAREST_EVEN);
+    EXPECT(mem[2] == 0.0f && mem[3] == 1.5f);
+    mem = {1.0f, 1.0f, -3.0f, 2.5f};
+    calculator.doMemoryWrite(m, o, MME_HIP_REDUCTION_MIN);
+    EXPECT(mem[0] == 5.9604645e-08f && mem[2] == -3.0f && mem[3] == -1.0f);
+    // bf16 sub: 1 - 2^-9 needs a ninth significant bit: nearest even gives 1, toward zero the bf16 below 1
+    std::vector<uint16_t> m16 = {bf16_of(1.0f), bf16_of(1.0f)}, o16 = {bf16_of(0.001953125f), bf16_of(0.001953125f)};
+    auto                  mb = std::make_shared<Tensor>(SizeArray {2, 1, 1, 1, 1}, 1, MME_HIP_BF16, m16.data());
+    auto                  ob = std::make_shared<Tensor>(SizeArray {2, 1, 1, 1, 1}, 1, MME_HIP_BF16, o16.data());
+    calculator.doMemoryWrite(mb, ob, MME_HIP_REDUCTION_SUB, MME_HIP_REDUCTION_RM_NEAREST_EVEN);
+    EXPECT(float_of_bf16(m16[0]) == 1.0f);
+    m16 = {bf16_of(1.0f), bf16_of(1.0f)};
+    calculator.doMemoryWrite(mb, ob, MME_HIP_REDUCTION_SUB, MME_HIP_REDUCTION_RM_TO_ZERO);
+    EXPECT(float_of_bf16(m16[0]) == 0.99609375f);
+    // reduction none copies
+    calculator.doMemoryWrite(mb, ob);
+    EXPECT(m16[0] == o16[0] && m16[1] == o16[1]);
+}
+
 // error conventions: what MME_ASSERT rejects must throw (mme_reference_impl.cpp:465-467, 591)
 static void error_conventions(Calculator& calculator)
 {
@@ -183,6 +216,7 @@ int main()
                      {"reference_gemm_2d_test_bf16", reference_gemm_2d_test_bf16},
                      {"fp8_convert", fp8_convert},
                      {"reference_gemm_simple_test_fp8", reference_gemm_simple_test_fp8},
+                     {"memory_write_reductions", memory_write_reductions},
                      {"error_conventions", error_conventions}};
         for (auto& c : cases)
         {

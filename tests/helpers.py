@@ -76,3 +76,37 @@ def cast_sweep_inputs():
 
 # relative Frobenius tolerances of the contraction against the reference's fp32-accumulated result
 TOL = {abi.BF16: 2e-3, abi.FP32: 2e-3, abi.FP8_143: 1e-2, abi.FP8_152: 1e-2}
+
+
+def rmw_operands(rng, dt, n):
+    """Pairs that exercise the adder: random magnitudes over the whole exponent range, near-cancellation, exponent gaps
+    around the mantissa width (where the smaller operand turns into guard / sticky bits), denormals, zeros of both
+    signs, inf, NaN, values next to overflow."""
+    if dt == abi.FP32:
+        bits, man = np.uint32, 23
+        rand = lambda k: rng.integers(0, 2**32, k, dtype=np.uint64).astype(np.uint32)
+    else:
+        bits, man = np.uint16, 7
+        rand = lambda k: rng.integers(0, 2**16, k, dtype=np.uint64).astype(np.uint16)
+    a, b = rand(n), rand(n)
+    q = n // 8
+    # near-cancellation: same exponent, opposite sign, close mantissas
+    b[:q] = (a[:q] ^ (1 << (man + 8))) ^ rng.integers(0, 4, q).astype(bits)
+    # exponent gaps of man-2 .. man+4 with both signs
+    ea = rng.integers(40, 200, q)
+    gap = rng.integers(man - 2, man + 5, q)
+    sgn = rng.integers(0, 2, (2, q))
+    a[q:2 * q] = ((sgn[0] << (man + 8)) | (ea << man) | rng.integers(0, 1 << man, q)).astype(bits)
+    b[q:2 * q] = ((sgn[1] << (man + 8)) | ((ea - gap) << man) | rng.integers(0, 1 << man, q)).astype(bits)
+    # small exponents: results around the denormal range
+    a[2 * q:3 * q] = ((sgn[0] << (man + 8)) | (rng.integers(0, 4, q) << man) | rng.integers(0, 1 << man, q)).astype(bits)
+    b[2 * q:3 * q] = ((sgn[1] << (man + 8)) | (rng.integers(0, 4, q) << man) | rng.integers(0, 1 << man, q)).astype(bits)
+    # large exponents: overflow
+    a[3 * q:4 * q] = ((sgn[0] << (man + 8)) | (rng.integers(252, 256, q) << man) | rng.integers(0, 1 << man, q)).astype(bits)
+    b[3 * q:4 * q] = ((sgn[1] << (man + 8)) | (rng.integers(252, 256, q) << man) | rng.integers(0, 1 << man, q)).astype(bits)
+    specials = np.array([0, 1 << (man + 8), 0xFF << man, (0xFF << man) | (1 << (man + 8)), (0xFF << man) | 1, 1, (1 << man), (0xFE << man) | ((1 << man) - 1)],
+                        dtype=np.uint64).astype(bits)
+    k = len(specials)
+    a[4 * q:4 * q + k * k] = np.repeat(specials, k)
+    b[4 * q:4 * q + k * k] = np.tile(specials, k)
+    return a, b

@@ -27,7 +27,7 @@ def _declared():
 def test_header_declares_entry_points():
     names = _declared()
     for must in ("mme_hip_create", "mme_hip_destroy", "mme_hip_batch_gemm", "mme_hip_convolution", "mme_hip_activation",
-                 "mme_hip_memory_write", "mme_hip_batch_gemm_dev", "mme_hip_convolution_dev", "mme_hip_cast_from_fp32_dev",
+                 "mme_hip_memory_write", "mme_hip_memory_write_dev", "mme_hip_batch_gemm_dev", "mme_hip_convolution_dev", "mme_hip_cast_from_fp32_dev",
                  "mme_hip_cast_to_fp32_dev"):
         assert must in names
 
