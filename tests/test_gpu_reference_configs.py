@@ -1,0 +1,125 @@
+"""The reference's own Gaudi3 test configurations (mme/mme_verification/gaudi3/configs, kept as data under
+tests/golden/configs/gaudi3) through the harness seam: every test whose operation and types the calculator path covers
+and whose contraction the CPU checker can afford runs MmeTestManager::runReference's sequence (contraction -> doActivation
+-> doMemoryWrite) once on the GPU library and once on the oracle, on the same operands."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from intel_gaudi3_software_amd import MmeSimTensor, abi, harness
+from helpers import A, OracleCalculator, TOL, rel_frobenius
+
+pytestmark = pytest.mark.gpu
+
+CONFIG_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "configs", "gaudi3")
+MAX_FLOPS = 1.2e9  # per test, for the CPU checker
+
+
+def _key(t):
+    return (t["operation"], t["in_type"], t["in2_type"], t["out_type"], tuple(t["x_sizes"]), tuple(t["w_sizes"]), tuple(t["y_sizes"]),
+            tuple(t["x_strides"] or ()), tuple(t["w_strides"] or ()), tuple(t["y_strides"] or ()), tuple(t["padding"]),
+            tuple(t["conv_strides"]), tuple(t["dilation"]), t["fp8_bias_in"], t["fp8_bias_in2"], t["fp8_bias_out"], t["inf_nan_a"],
+            t["inf_nan_b"], t["inf_nan_out"], t["rounding"], t["reduction_op"], t["reduction_rm"], t["clip"], t["clip_inf_in"],
+            t["flush_denormals"], t["stochastic_flush"], t["relu"])
+
+
+def _collect():
+    cases, seen = [], set()
+    for path in sorted(glob.glob(os.path.join(CONFIG_DIR, "*", "*.json"))):
+        for i, t in enumerate(harness.load_tests(path, seed=7)):
+            if harness.supported(t) is not None or harness.contraction_flops(t) > MAX_FLOPS:
+                continue
+            k = _key(t)
+            if k in seen:  # tests that differ only in descriptor-generation parameters are one case for the calculator
+                continue
+            seen.add(k)
+            cases.append(pytest.param(t, id="%s-%d-%s" % (os.path.basename(path)[:-5], i, t["operation_name"])))
+    return cases
+
+
+def _quantise(orc, values, dtype, bias, mode):
+    out = np.zeros(values.size, abi.DTYPE_NUMPY[dtype])
+    if dtype == abi.FP32:
+        out[:] = values
+        return out
+    assert orc.orc_cast_from_fp32(out.ctypes.data, dtype, bias, mode, values.ctypes.data, values.size, 0, None, 0, 0, 0, 1, 0, 0) == 0
+    return out
+
+
+def _decode(orc, codes, dtype, bias, mode):
+    if dtype == abi.FP32:
+        return codes.view(np.float32).copy()
+    out = np.zeros(codes.size, np.float32)
+    assert orc.orc_cast_to_fp32(out.ctypes.data, codes.ctypes.data, dtype, bias, mode, codes.size, 0, None, 0) == 0
+    return out
+
+
+@pytest.mark.parametrize("t", _collect())
+def test_reference_config(calc, orc, t):
+    types = harness.tensor_types(t)
+    a_l, b_l, o_l = harness.operand_roles(t)
+    values = harness.make_operand_values(t, seed=11)
+    host = {}
+    for letter in (a_l, b_l):
+        dtype, bias, mode = types[letter]
+        # moderate magnitudes keep fp8 operands away from the formats' special codes, as the reference's generator does
+        v = values[letter]
+        if dtype in (abi.FP8_143, abi.FP8_152):
+            v = np.clip(v, -8.0, 8.0)
+        host[letter] = _quantise(orc, v.astype(np.float32), dtype, bias, mode)
+    mk = lambda letter: MmeSimTensor(t[letter + "_sizes"], 5, types[letter][0], host[letter].copy(), types[letter][1], types[letter][2],
+                                     t[letter + "_strides"])
+    out_dtype, out_bias, out_mode = types[o_l]
+    n_out = max(st * sz for st, sz in zip(MmeSimTensor(t[o_l + "_sizes"], 5, out_dtype, None, out_bias, out_mode, t[o_l + "_strides"]).strides,
+                                          t[o_l + "_sizes"] + [1] * 5))
+    prev = None
+    if t["reduction_op"] != abi.REDUCTION_NONE:
+        rng = np.random.default_rng(5)
+        prev = _quantise(orc, rng.uniform(-4, 4, n_out).astype(np.float32), out_dtype, out_bias, out_mode)
+    lfsr = (np.arange(256, dtype=np.uint32) * 2654435761 + 12345).astype(np.uint32)
+    poly = 0xB4BCD35C
+    from intel_gaudi3_software_amd import HipCalculator
+    gpu = HipCalculator(lfsrNumRegs=256, lfsr=lfsr, polynomial=poly) if t["uses_lfsr"] else calc
+    cpu = OracleCalculator(orc, lfsr, poly)
+    results = []
+    for c in (gpu, cpu):
+        tensors = {a_l: mk(a_l), b_l: mk(b_l)}
+        p = None if prev is None else MmeSimTensor(t[o_l + "_sizes"], 5, out_dtype, prev.copy(), out_bias, out_mode, t[o_l + "_strides"])
+        results.append(harness.run_reference_sequence(c, t, tensors, p).data())
+    if gpu is not calc:
+        gpu.close()
+    got, want = (_decode(orc, np.ascontiguousarray(r), out_dtype, out_bias, out_mode) for r in results)
+    fin = np.isfinite(want)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+    # the accumulators differ in the last bits (IEEE FMA order on the GPU, the Gaudi3 truncating tree in the reference), so
+    # a rounded output may land on the neighbouring code; stochastic modes amplify that to one code wherever the draw falls
+    # between the two accumulators
+    tol = 3e-2 if (t["uses_lfsr"] or out_dtype in (abi.FP8_143, abi.FP8_152)) else max(TOL[t["in_type"]], 4e-3 if out_dtype == abi.BF16 else 0)
+    assert rel_frobenius(got[fin], want[fin]) <= tol
+    if out_dtype != abi.FP32:  # (fp32 outputs are the accumulators themselves)
+        same = np.mean(results[0] == results[1])
+        # (0.8: the longest reductions of the set, 10^5 products, let the tree's truncation reach a quarter of a bf16 ulp)
+        assert same >= (0.5 if t["uses_lfsr"] else 0.8), same
+
+
+def test_external_reference_protocol(calc, orc, tmp_path):
+    """inputA.bin / inputB.bin -> mme_output.bin (mme_test_data_gen.cpp:561-573, mme_test_manager.cpp:586-611) equals the
+    sequence run on tensors directly, byte for byte."""
+    t = harness.load_tests(os.path.join(CONFIG_DIR, "basic_tests", "basic_fwd.json"))[0]
+    assert harness.supported(t) is None
+    types = harness.tensor_types(t)
+    a_l, b_l, o_l = harness.operand_roles(t)
+    values = harness.make_operand_values(t, seed=3)
+    host = {letter: _quantise(orc, values[letter], *types[letter]) for letter in (a_l, b_l)}
+    host[a_l].tofile(str(tmp_path / "inputA.bin"))
+    host[b_l].tofile(str(tmp_path / "inputB.bin"))
+    got = harness.run_ext_ref(t, str(tmp_path), calc)
+    dumped = np.fromfile(str(tmp_path / "mme_output.bin"), dtype=got.dtype)
+    tensors = {letter: MmeSimTensor(t[letter + "_sizes"], 5, types[letter][0], host[letter].copy(), types[letter][1], types[letter][2],
+                                    t[letter + "_strides"]) for letter in (a_l, b_l)}
+    want = harness.run_reference_sequence(calc, t, tensors).data()
+    assert np.array_equal(dumped, want) and np.array_equal(got, want)
+    assert np.any(want != 0)
