@@ -526,7 +526,7 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
 {
     if (!h) return MME_HIP_EINVAL;
     if (!cp) return fail(h, MME_HIP_EINVAL, "got null pointer");
-    if (op == MME_HIP_OP_DETERMINISTIC_DEDW) return fail(h, MME_HIP_EUNSUPPORTED, "op %d is not built in this library", op);
+    // (deterministic_dedw is a descriptor-generation variant: the reference's calculator rejects it too, mme_reference_impl.cpp:656-657)
     if (op == MME_HIP_OP_TRANSPOSED_DEDX)
     {
         // mme_reference_impl.cpp:625-647: exchange the first two weight dimensions, reverse the S axis, then dedx.  The
