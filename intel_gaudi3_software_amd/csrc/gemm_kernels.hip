@@ -137,7 +137,7 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s)
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     if (p.M <= 0 || p.N <= 0 || nb <= 0) return hipSuccess;
     hipError_t e;
-    if (gemm_fp8_fast_applicable(p)) e = launch_gemm_fp8_fast(p, s);
+    if (gemm_large_tile_applicable(p)) e = launch_gemm_large_tile(p, s);
     else
     {
         const int tiles = ((p.M + TILE - 1) / TILE) * ((p.N + TILE - 1) / TILE);

@@ -1,4 +1,4 @@
-// gemm_fp8_fast.hip -- the contraction for large aligned problems (the headline path: fp8_143 / fp8_152 operands, and
+// gemm_large_tile.hip -- the contraction for large aligned problems (the headline path: fp8_143 / fp8_152 operands, and
 // bf16 through the same code; M and N multiples of 256, K a multiple of 128 bytes and >= 384 bytes, 16-byte aligned rows).
 //
 // Same arithmetic as the general kernel (gemm_impl.hpp): OCP fp8 (or bf16) MFMA with fp32 accumulation, Gaudi's exponent
@@ -766,7 +766,7 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 }
 } // namespace
 
-bool gemm_fp8_fast_applicable(const GemmProblem& p)
+bool gemm_large_tile_applicable(const GemmProblem& p)
 {
     if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152 || p.dtype == DT_BF16)) return false;
     const int es = p.dtype == DT_BF16 ? 2 : 1;
@@ -820,7 +820,7 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
 {
     GemmProblem q = p;
     q.split_k = 1;
-    if (!gemm_fp8_fast_applicable(q)) return 0;
+    if (!gemm_large_tile_applicable(q)) return 0;
     const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
     const int       nk = p.K * (p.dtype == DT_BF16 ? 2 : 1) / FBK;
     int             best = 1;
@@ -845,7 +845,7 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
     return best;
 }
 
-hipError_t launch_gemm_fp8_fast(const GemmProblem& p, hipStream_t s)
+hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     dim3            grid(((p.M + FBM - 1) / FBM) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);

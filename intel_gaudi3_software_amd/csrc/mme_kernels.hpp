@@ -101,10 +101,10 @@ struct GemmProblem
 size_t     gemm_workspace_bytes(const GemmProblem& p);
 int        gemm_pick_split_k(const GemmProblem& p, int num_cus);
 hipError_t launch_gemm(const GemmProblem& p, hipStream_t s);
-// large aligned fp8 problems (gemm_fp8_fast.hip); launch_gemm routes to it when applicable
-bool       gemm_fp8_fast_applicable(const GemmProblem& p);
+// large aligned fp8 problems (gemm_large_tile.hip); launch_gemm routes to it when applicable
+bool       gemm_large_tile_applicable(const GemmProblem& p);
 int        gemm_fast_pick_split_k(const GemmProblem& p, int num_cus); // 0: the large-tile kernel does not take this problem
-hipError_t launch_gemm_fp8_fast(const GemmProblem& p, hipStream_t s);
+hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s);
 
 // forward convolution fast path (conv_fwd_fast.hip): bf16, 3x3, 64 -> 64 channels, stride 1, padding 1, dense NHWC
 bool       conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int W, int H, int D, const int stride[4], const int dil[4],
