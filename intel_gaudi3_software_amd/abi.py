@@ -17,7 +17,7 @@ OK, EINVAL, EUNSUPPORTED, EHIP, ENOMEM = 0, -1, -2, -3, -4
 # ChipType
 CHIP_GAUDI, CHIP_GAUDI2, CHIP_GAUDI3 = 0, 1, 2
 # EMmeDataType
-FP8_143, FP8_152, FP16, BF16, FP32, FP32_IEEE, TF32 = 9, 10, 11, 12, 13, 14, 15
+FP8_143, FP8_152, FP16, BF16, FP32, FP32_IEEE, TF32, UFP16 = 9, 10, 11, 12, 13, 14, 15, 17
 # RoundingMode
 RM_NEAREST_EVEN, RM_TO_ZERO, RM_UP, RM_DOWN, RM_STOCHASTIC, RM_HALF_AWAY, RM_STOCHASTIC_AND_NEAREST = 0, 1, 2, 3, 4, 6, 7
 # EMmeOpType
@@ -27,10 +27,10 @@ FULL_INF_NAN, NO_INF_NAN, MINIMAL_INF_NAN = 0, 1, 2
 REDUCTION_ADD, REDUCTION_SUB, REDUCTION_MIN, REDUCTION_MAX, REDUCTION_MAX_0, REDUCTION_NONE = range(6)  # EMmeReductionOp
 FP8_SPECIALS_CHECK, FP8_SPECIALS_ASSUME_NONE = 0, 1
 
-DTYPE_SIZE = {FP8_143: 1, FP8_152: 1, FP16: 2, BF16: 2, FP32: 4, FP32_IEEE: 4, TF32: 4}
-DTYPE_NUMPY = {FP8_143: np.uint8, FP8_152: np.uint8, BF16: np.uint16, FP16: np.uint16, FP32: np.float32,
+DTYPE_SIZE = {FP8_143: 1, FP8_152: 1, FP16: 2, UFP16: 2, BF16: 2, FP32: 4, FP32_IEEE: 4, TF32: 4}
+DTYPE_NUMPY = {FP8_143: np.uint8, FP8_152: np.uint8, BF16: np.uint16, FP16: np.uint16, UFP16: np.uint16, FP32: np.float32,
                FP32_IEEE: np.float32, TF32: np.uint32}
-DTYPE_NAME = {FP8_143: "fp8_143", FP8_152: "fp8_152", BF16: "bf16", FP16: "fp16", FP32: "fp32",
+DTYPE_NAME = {FP8_143: "fp8_143", FP8_152: "fp8_152", BF16: "bf16", FP16: "fp16", UFP16: "ufp16", FP32: "fp32",
               FP32_IEEE: "fp32_ieee", TF32: "tf32"}
 
 

@@ -411,7 +411,7 @@ int mme_hip_create(mme_hip_handle* out, int chip, int max_tensor_dims, int max_c
         h->polynomial = (uint32_t) distr(gen);
     }
     else
-        h->polynomial = polynomial;
+        h->polynomial = polynomial & 0xFFFFu; // the reference keeps it in a uint16_t member (mme_reference_impl.h:253)
     *out = h;
     return MME_HIP_OK;
 }

@@ -72,6 +72,22 @@ def oracle():
         L.orc_add_fp32_n.argtypes = [vp, vp, vp, C.c_size_t, C.c_int]
         L.orc_tree9_n.argtypes = [vp, vp, vp, C.c_size_t, C.c_int]
         L.orc_memory_write.argtypes = [vp, vp, C.c_int, C.c_int, C.c_int]
+        L.orc_cfp16_to_fp32.restype = C.c_uint32
+        L.orc_cfp16_to_fp32.argtypes = [C.c_uint16, C.c_int, C.c_int, C.c_int]
+        L.orc_fp32_to_cfp16.restype = C.c_uint16
+        L.orc_fp32_to_cfp16.argtypes = [C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_uint32] + [C.c_int] * 4
+        L.orc_fp32_to_tf32.restype = C.c_uint32
+        L.orc_fp32_to_tf32.argtypes = [C.c_uint32, C.c_int, C.c_int]
+        L.orc_fma_vec_fp16.restype = C.c_uint32
+        L.orc_fma_vec_fp16.argtypes = [vp, C.c_ssize_t, C.c_int, C.c_int, C.c_int, vp, C.c_ssize_t, C.c_int, C.c_int,
+                                       C.c_int, C.c_size_t]
+        L.orc_fma_vec_tf32.restype = C.c_uint32
+        L.orc_fma_vec_tf32.argtypes = [vp, C.c_ssize_t, vp, C.c_ssize_t, C.c_size_t, C.c_int, C.c_int]
+        L.orc_batch_gemm_clip.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int]
+        L.orc_convolution_clip.argtypes = [vp, vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.orc_fp32_to_cfp16_n.argtypes = [vp, vp, C.c_size_t, C.c_int, C.c_int, C.c_int, vp] + [C.c_int] * 4
+        L.orc_cfp16_to_fp32_n.argtypes = [vp, vp, C.c_size_t, C.c_int, C.c_int, C.c_int]
+        L.orc_fp32_to_tf32_n.argtypes = [vp, vp, C.c_size_t, C.c_int, C.c_int]
         _oracle = L
     return _oracle
 
@@ -98,6 +114,12 @@ def ref():
         L.ref_tree9_n.argtypes = [vp, vp, vp, C.c_size_t, C.c_int]
         L.ref_fma_vec.restype = C.c_uint32
         L.ref_fma_vec.argtypes = [vp, vp, C.c_uint, C.c_int, C.c_int, C.c_uint, C.c_uint, C.c_int, C.c_int]
+        L.ref_fma_vec_clip.restype = C.c_uint32
+        L.ref_fma_vec_clip.argtypes = [vp, vp, C.c_uint, C.c_int, C.c_int, C.c_uint, C.c_uint] + [C.c_int] * 4
+        L.ref_batch_gemm_clip.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int]
+        L.ref_fp32_to_cfp16_n.argtypes = [vp, vp, C.c_size_t, C.c_int, C.c_int, C.c_int, vp] + [C.c_int] * 4
+        L.ref_cfp16_to_fp32_n.argtypes = [vp, vp, C.c_size_t, C.c_int, C.c_int, C.c_int]
+        L.ref_fp32_to_tf32_n.argtypes = [vp, vp, C.c_size_t, C.c_int, C.c_int]
         _ref = L
     return _ref
 
