@@ -191,6 +191,8 @@ public:
     void  setStream(void* hipStream) { check(mme_hip_set_stream(m_h, hipStream)); }
     void  synchronize() { check(mme_hip_synchronize(m_h)); }
     void  setFp8SpecialsPolicy(int policy) { check(mme_hip_set_fp8_specials_policy(m_h, policy)); }
+    /* clipFp / clipFpInfIn for the device-resident contractions (read by the tf32 operand conversion only) */
+    void  setOperandClip(bool clipFp, bool clipFpInfIn) { check(mme_hip_set_operand_clip(m_h, clipFp, clipFpInfIn)); }
     mme_hip_handle handle() const { return m_h; }
 
 private:

@@ -145,6 +145,7 @@ class HipCalculator:
         rc = self._lib.mme_hip_create(C.byref(self._h), chip, max_tensor_dims, max_conv_dims, seed, lfsrNumRegs, lf, polynomial)
         if rc != 0:
             raise MMEStackException(self._lib.mme_hip_last_error(None).decode(), rc)
+        self._caller_stream = False
 
     def close(self):
         if getattr(self, "_h", None) is not None and self._h.value:
@@ -169,6 +170,7 @@ class HipCalculator:
                     epilogue=None):
         dev = self._placement(outputTensor, xTensor, wTensor)
         if dev:
+            self._check(self._lib.mme_hip_set_operand_clip(self._h, int(clipFp), int(clipFpInfIn)))
             self._check(self._lib.mme_hip_batch_gemm_dev(self._h, outputTensor.desc, xTensor.desc, wTensor.desc, op,
                                                          epilogue.pod if epilogue else None))
         else:
@@ -182,6 +184,7 @@ class HipCalculator:
         dev = self._placement(outputTensor, xTensor, wTensor, yTensor)
         pod = params.pod()
         if dev:
+            self._check(self._lib.mme_hip_set_operand_clip(self._h, int(clipFp), int(clipFpInfIn)))
             self._check(self._lib.mme_hip_convolution_dev(self._h, outputTensor.desc, xTensor.desc, wTensor.desc, yTensor.desc,
                                                           pod, op, epilogue.pod if epilogue else None))
         else:
@@ -213,7 +216,21 @@ class HipCalculator:
         return self._lib.mme_hip_stream(self._h)
 
     def setStream(self, hip_stream):
+        """Enqueue on a caller-owned stream (0 / None: back to the calculator's own).  With a caller-owned stream the
+        ordering against the producers of the operands is the caller's business; on its own stream the calculator waits,
+        on the device, for what torch's current stream has enqueued so far before every call on torch tensors."""
         self._check(self._lib.mme_hip_set_stream(self._h, hip_stream))
+        self._caller_stream = bool(hip_stream)
+
+    def _after_torch(self):
+        # the calculator's own stream does not synchronise with any other: make it wait (on the device) for the fills and
+        # copies that produced the operands on torch's current stream
+        if self._caller_stream:
+            return
+        import torch
+        ev = torch.cuda.Event()
+        ev.record()
+        torch.cuda.ExternalStream(self.stream()).wait_event(ev)
 
     def setFp8SpecialsPolicy(self, policy):
         self._check(self._lib.mme_hip_set_fp8_specials_policy(self._h, policy))
@@ -221,6 +238,7 @@ class HipCalculator:
     def castFromFp32(self, out, out_dtype, src, n, fpBias=0, infNanMode=FULL_INF_NAN, scale_exp=0, col_scale_exp=None,
                      n_cols=0, relu=False, rm=RM_NEAREST_EVEN, clipFp=False, clipInfIn=False, flushDenorms=False):
         """Flat quantise / cast on device buffers (torch tensors)."""
+        self._after_torch()
         self._check(self._lib.mme_hip_cast_from_fp32_dev(
             self._h, out.data_ptr(), out_dtype, fpBias, infNanMode, src.data_ptr(), n, scale_exp,
             col_scale_exp.data_ptr() if col_scale_exp is not None else None, n_cols, int(relu), rm, int(clipFp), int(clipInfIn),
@@ -228,16 +246,19 @@ class HipCalculator:
 
     def castToFp32(self, out, src, in_dtype, n, fpBias=0, infNanMode=FULL_INF_NAN, scale_exp=0, col_scale_exp=None, n_cols=0):
         """Flat dequantise on device buffers (torch tensors)."""
+        self._after_torch()
         self._check(self._lib.mme_hip_cast_to_fp32_dev(
             self._h, out.data_ptr(), src.data_ptr(), in_dtype, fpBias, infNanMode, n, scale_exp,
             col_scale_exp.data_ptr() if col_scale_exp is not None else None, n_cols))
 
     def absmax(self, out, src, n):
+        self._after_torch()
         self._check(self._lib.mme_hip_absmax_dev(self._h, out.data_ptr(), src.data_ptr(), n))
 
-    @staticmethod
-    def _placement(*tensors):
+    def _placement(self, *tensors):
         dev = [t.is_device for t in tensors]
         if any(dev) and not all(dev):
             raise MMEStackException("tensors of one call must all be host or all be device resident", abi.EINVAL)
+        if all(dev):
+            self._after_torch()
         return all(dev)

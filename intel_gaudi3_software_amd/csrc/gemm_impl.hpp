@@ -11,7 +11,7 @@
 // 64 bytes of the reduction dimension per LDS stage, two stages (loads of stage i+1 are in flight while stage i feeds
 // the matrix cores).  Every lane reads a 32-byte k-slab per row and stage:
 //     fp8  : one v_mfma_f32_32x32x64_f8f6f4 (e4m3 / e5m2 selectable per operand)
-//     bf16 : two v_mfma_f32_32x32x16_bf16
+//     bf16 : two v_mfma_f32_32x32x16_bf16 (fp16: the same with v_mfma_f32_32x32x16_f16)
 //     fp32 : eight v_mfma_f32_32x32x2_f32
 // LDS rows are k-contiguous for both operands (row pitch 80 B: conflict-free 16-byte reads); operands whose memory
 // layout is contiguous along the free index (B of the "ab" form, x of dedw, ...) are transposed in registers with
@@ -30,6 +30,7 @@ typedef int   v8i __attribute__((ext_vector_type(8)));
 typedef int   v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 // Kernel arguments are read in place from the kernarg segment (constant address space): views are passed on by
 // reference to out-of-line helpers without a private copy of the whole problem, and uniform fields stay scalar loads.
@@ -303,13 +304,23 @@ __device__ __forceinline__ void mma_slab(v16f& acc, const Slab& a, const Slab& b
         {
             uint4 u;
             v8bf  v;
+            v8h   h;
         } a0, a1, b0, b1;
         a0.u = a.lo;
         a1.u = a.hi;
         b0.u = b.lo;
         b1.u = b.hi;
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, b0.v, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, b1.v, acc, 0, 0, 0);
+        if constexpr (FMT == 1)
+        {
+            // IEEE half operands
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0.h, b0.h, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1.h, b1.h, acc, 0, 0, 0);
+        }
+        else
+        {
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0.v, b0.v, acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1.v, b1.v, acc, 0, 0, 0);
+        }
     }
     else
     {
@@ -323,6 +334,13 @@ __device__ __forceinline__ void mma_slab(v16f& acc, const Slab& a, const Slab& b
 // ------------------------------------------------------------------------------------------------------------
 // epilogue: alpha, per-column power of two, relu, cast, store
 // ------------------------------------------------------------------------------------------------------------
+// fp16 / ufp16 outputs: one out-of-line copy of the converter, so that the unrolled epilogues of the other output types
+// keep their size
+__device__ __attribute__((noinline)) uint32_t cast_half_out_of_line(float v, const CastParams& cp)
+{
+    return cp.dtype == DT_UFP16 ? cast_elem<DT_UFP16, false>(v, cp) : cast_elem<DT_FP16, false>(v, cp);
+}
+
 __device__ __forceinline__ void store_out(EpilogueRef e, long long idx, float v)
 {
     if (!e.fused)
@@ -343,6 +361,8 @@ __device__ __forceinline__ void store_out(EpilogueRef e, long long idx, float v)
         case DT_BF16:
             ((uint16_t*) e.out)[idx] = (uint16_t) (e.fast_cast ? cast_elem<DT_BF16, true>(v, cp) : cast_elem<DT_BF16, false>(v, cp));
             break;
+        case DT_FP16:
+        case DT_UFP16: ((uint16_t*) e.out)[idx] = (uint16_t) cast_half_out_of_line(v, cp); break;
         default: ((uint32_t*) e.out)[idx] = cast_elem<DT_FP32, false>(v, cp); break;
     }
 }

@@ -6,6 +6,7 @@ namespace mme
 {
 // one translation unit per operand type / fp8 flavour pair keeps the build parallel
 void launch_gemm_bf16(const GemmProblem& p, dim3 grid, hipStream_t s);
+void launch_gemm_fp16(const GemmProblem& p, dim3 grid, hipStream_t s);
 void launch_gemm_fp32(const GemmProblem& p, dim3 grid, hipStream_t s);
 void launch_gemm_fp8_00(const GemmProblem& p, dim3 grid, hipStream_t s);
 void launch_gemm_fp8_10(const GemmProblem& p, dim3 grid, hipStream_t s);
@@ -123,7 +124,7 @@ int gemm_pick_split_k(const GemmProblem& p, int num_cus)
     if (const int fast = gemm_fast_pick_split_k(p, num_cus)) return fast; // the large-tile kernel takes this problem
     // split the reduction only when the output tiles cannot fill the chip and the reduction is long
     const long long tiles = (long long) ((p.M + TILE - 1) / TILE) * ((p.N + TILE - 1) / TILE) * p.batch[0] * p.batch[1] * p.batch[2];
-    const int       es = (p.dtype == DT_BF16) ? 2 : (p.dtype == DT_FP32 ? 4 : 1);
+    const int       es = dt_bytes(p.dtype);
     const int       nk = (p.K + STAGE_BYTES / es - 1) / (STAGE_BYTES / es);
     if (tiles >= num_cus || nk < 16) return 1;
     long long s = (2LL * num_cus + tiles - 1) / tiles;
@@ -145,6 +146,7 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s)
         switch (p.dtype)
         {
             case DT_BF16: launch_gemm_bf16(p, grid, s); break;
+            case DT_FP16: launch_gemm_fp16(p, grid, s); break;
             case DT_FP32: launch_gemm_fp32(p, grid, s); break;
             case DT_FP8_143:
             case DT_FP8_152:

@@ -808,6 +808,7 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     if (p.epi.ld <= 0) return false;
     {
         const int out_dt = p.epi.fused ? p.epi.out_dtype : DT_FP32;
+        if (out_dt == DT_FP16 || out_dt == DT_UFP16) return false; // these outputs take the general kernel's epilogue
         const int per16 = out_dt == DT_FP32 ? 4 : (out_dt == DT_BF16 ? 8 : 16); // elements per 16 bytes
         if ((p.epi.ld % per16) || ((uintptr_t) p.epi.out & 15)) return false;
         for (int d = 0; d < 3; d++)

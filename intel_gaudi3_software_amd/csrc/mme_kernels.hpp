@@ -28,6 +28,8 @@ hipError_t launch_repack_transposed_weights(void* out, const void* in, int elem_
 // zero, 2 up, 3 down)
 hipError_t launch_memory_write_reduce(void* memory, const void* mme_out, int dtype, size_t n, int op, int rm, int clip, hipStream_t s);
 hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s);
+// fp32 words -> the same words rounded to tf32 (nearest even, 10 mantissa bits), out of place
+hipError_t launch_round_to_tf32(void* out, const void* in, size_t n, int clip, int clip_inf_in, hipStream_t s);
 hipError_t launch_absmax(float* out, const float* in, size_t n, hipStream_t s);
 
 // ---- contraction (gemm_kernels.hip) ---------------------------------------------------------------------------

@@ -75,7 +75,7 @@ def cast_sweep_inputs():
 
 
 # relative Frobenius tolerances of the contraction against the reference's fp32-accumulated result
-TOL = {abi.BF16: 2e-3, abi.FP32: 2e-3, abi.FP8_143: 1e-2, abi.FP8_152: 1e-2}
+TOL = {abi.BF16: 2e-3, abi.FP32: 2e-3, abi.FP8_143: 1e-2, abi.FP8_152: 1e-2, abi.FP16: 2e-3, abi.UFP16: 2e-3, abi.TF32: 2e-3}
 
 
 def rmw_operands(rng, dt, n):
@@ -125,11 +125,11 @@ class OracleCalculator:
         assert rc == 0, self.orc.orc_last_error()
 
     def doBatchGemm(self, out, x, w, op, rm=0, clipFp=False, clipFpInfIn=False, zeroPoints=None):
-        self._ok(self.orc.orc_batch_gemm(A(out.desc), A(x.desc), A(w.desc), op))
+        self._ok(self.orc.orc_batch_gemm_clip(A(out.desc), A(x.desc), A(w.desc), op, int(clipFp), int(clipFpInfIn)))
 
     def doConvolution(self, out, x, w, y, params, op, rm=0, clipFp=False, clipFpInfIn=False, zeroPoints=None):
         p = params.pod()
-        self._ok(self.orc.orc_convolution(A(out.desc), A(x.desc), A(w.desc), A(y.desc), A(p), op, rm))
+        self._ok(self.orc.orc_convolution_clip(A(out.desc), A(x.desc), A(w.desc), A(y.desc), A(p), op, rm, int(clipFp), int(clipFpInfIn)))
 
     def doActivation(self, output, acc, res=None, bias=None, relu=False, rm=0, actParams=None, clipFp=False, clipInfIn=False,
                      flushDenorms=False, stochasticFTZfp8=False):

@@ -44,6 +44,8 @@ def _quantise(orc, values, dtype, bias, mode):
     if dtype == abi.FP32:
         out[:] = values
         return out
+    if dtype == abi.TF32:  # fp32 words; the contraction rounds them on entry
+        return values.view(np.uint32).copy()
     assert orc.orc_cast_from_fp32(out.ctypes.data, dtype, bias, mode, values.ctypes.data, values.size, 0, None, 0, 0, 0, 1, 0, 0) == 0
     return out
 
