@@ -78,6 +78,9 @@ class MmeSimTensor:
     def data(self):
         return self._keep
 
+    def getDim(self):
+        return self.dim
+
     def getSizes(self):
         return list(self.sizes)
 

@@ -29,655 +29,12 @@
 //
 // Replaces, for these shapes, doGemmWorkerFloat + Gaudi3Fp8Fma::fma_vec of the reference
 // (mme/mme_reference/mme_reference_impl.cpp:1022-1053, chip_fma/gaudi3_fma.cpp:70-144).
-#include <type_traits>
-
-#include "gemm_impl.hpp"
+#include "gemm_large_tile_impl.hpp"
 
 namespace mme
 {
 namespace
 {
-typedef int v2i __attribute__((ext_vector_type(2)));
-#define LDS3 __attribute__((address_space(3)))
-
-constexpr int FBM = 256, FBN = 256, FBK = 64, FNST = 4;
-constexpr int FSTAGE = FBM * FBK + FBK * FBN; // 32 KiB
-
-__device__ __forceinline__ int fa_pos(int r, int c) { return r * 4 + (c ^ ((r >> 2) & 3)); }
-__device__ __forceinline__ int fb_pos(int k, int cb) { return k * 16 + ((cb + 2 * (k & 7)) & 15); }
-
-// 16 bytes per lane from global memory to LDS at lds_off + lane * 16 (lds_off is wave-uniform).  Inline assembly keeps
-// the request out of the compiler's memory model: it would otherwise order every later LDS read behind it.
-__device__ __forceinline__ void dma16(const void* g, uint32_t lds_off)
-{
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_off) : "memory");
-}
-
-struct Frags
-{
-    v8i a[4], b[2];
-};
-
-__device__ __forceinline__ void read_a(Frags& f, int i, const char* st, int wm, int lane)
-{
-    const int r = wm * 128 + i * 32 + (lane & 31), c0 = 2 * (lane >> 5);
-    const v4i lo = *(const v4i*) (st + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + fa_pos(r, c0 + 1) * 16);
-    f.a[i] = v8i {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-}
-
-// B stored n-contiguous: transposed LDS reads
-__device__ __forceinline__ void read_b_tr(Frags& f, int j, const char* st, int wn, int lane)
-{
-    const int q = lane >> 4, cb = wn * 4 + j * 2 + (q & 1), g = q >> 1, rr = (lane & 15) >> 1, h = lane & 1;
-    v2i       t[4];
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++)
-    {
-        const int k = g * 32 + 8 * tt + rr;
-        t[tt] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS3 v2i*) (st + FBM * FBK + fb_pos(k, cb) * 16 + h * 8));
-    }
-    f.b[j] = v8i {t[0].x, t[0].y, t[1].x, t[1].y, t[2].x, t[2].y, t[3].x, t[3].y};
-}
-
-// bf16, B stored n-contiguous: a stage is 32 k-rows x 256 columns x 2 B = 32 chunks of 16 B per row, the 32-byte blocks of a
-// row XOR-swizzled by k & 3.  ds_read_b64_tr_b16: within a group of 16 lanes, lane q addresses the 8-byte piece q % 4 of
-// row q / 4 and receives 4 consecutive k of its own column.  The fragment's k order ({0-7, 16-23} then {8-15, 24-31}
-// for the two lane halves) is the one the k-contiguous reads of the other operand produce.
-__device__ __forceinline__ void read_b_tr16(Frags& f, int j, const char* st, int wn, int lane)
-{
-    typedef short v4s __attribute__((ext_vector_type(4)));
-    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wn * 4 + j * 2 + (g & 1);
-    union
-    {
-        v4s h4[4];
-        v8i v;
-    } u;
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++)
-    {
-        // reads 0, 1 -> k = 16 h + 0 .. 7 (first MFMA), reads 2, 3 -> k = 16 h + 8 .. 15 (second MFMA)
-        const int k = 16 * h + 4 * tt + (q >> 2);
-        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + FBM * FBK + k * 512 + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
-    }
-    f.b[j] = u.v;
-}
-
-// bf16, A stored f-contiguous: the same stage layout and reads as an n-contiguous B, over the wavefront's 128 rows
-__device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int wm, int lane)
-{
-    typedef short v4s __attribute__((ext_vector_type(4)));
-    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wm * 8 + i * 2 + (g & 1);
-    union
-    {
-        v4s h4[4];
-        v8i v;
-    } u;
-#pragma unroll
-    for (int tt = 0; tt < 4; tt++)
-    {
-        const int k = 16 * h + 4 * tt + (q >> 2);
-        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + k * 512 + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
-    }
-    f.a[i] = u.v;
-}
-
-// B stored k-contiguous (the "abt" form): same layout and reads as A
-__device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int wn, int lane)
-{
-    const int r = wn * 64 + j * 32 + (lane & 31), c0 = 2 * (lane >> 5);
-    const v4i lo = *(const v4i*) (st + FBM * FBK + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + FBM * FBK + fa_pos(r, c0 + 1) * 16);
-    f.b[j] = v8i {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-}
-
-#define FENCE __builtin_amdgcn_sched_barrier(0)
-
-// ES = 1: fp8 (FMT selects e4m3 / e5m2 per operand), ES = 2: bf16.  Everything up to the matrix-core instruction is
-// byte-based and shared: a stage is 64 bytes of k per row for both.
-// GATHER: A is a convolution view with pixels along f (im2col addressing of mme/mme_reference/im2col.cpp:134-172 for the
-// forward pass, its gather-form inverse for dedx): row r of the tile is a pixel, a 64-byte stage is a run of channels
-// of one filter tap, so a request's address is (pixel's offset for tap 0) + (the tap's uniform offset) + channel, or a
-// page of zeros where the tap falls outside the source tensor.  B may then be a tapped weight view (dedx).
-__device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
-
-//
-// AMODE says how operand A is addressed: 0 plain, k contiguous; 1 convolution view with pixels along f (GATHER above);
-// 2 plain, f contiguous (the "atb" forms; bf16 only: the stage then holds 32 k-rows x 256 f like an n-contiguous B and is
-// read with ds_read_b64_tr_b16); 3 convolution view with pixels along k (dedw: f = tap * channels + channel is fixed per
-// lane, the pixel advances by 32 per stage and is decoded incrementally).
-template<int ES, int FMT, bool B_KC, int AMODE = 0>
-__device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
-{
-    constexpr bool GATHER = AMODE == 1;           // tap masks + uniform tap offsets
-    constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3; // the last row tile may be partial
-    constexpr bool A_KC = AMODE < 2;
-    extern __shared__ __attribute__((aligned(1024))) char lds[];
-    if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
-
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
-    const int tiles_n = g.N / FBN, tiles_m = (g.M + FBM - 1) / FBM;
-    int       tm, tn;
-    {
-        const int b = blockIdx.x, T = tiles_m * tiles_n;
-        if ((tiles_m % 8 == 0) && (tiles_n % 4 == 0))
-        {
-            const int L = (b & 7) * (T >> 3) + (b >> 3), Bx = L >> 5, w = L & 31, nbn = tiles_n >> 2;
-            tm = (Bx / nbn) * 8 + (w >> 2);
-            tn = (Bx % nbn) * 4 + (w & 3);
-        }
-        else
-        {
-            tm = b / tiles_n;
-            tn = b % tiles_n;
-        }
-    }
-    int       bz = blockIdx.y;
-    const int b0 = bz % g.batch[0];
-    bz /= g.batch[0];
-    const int       b1 = bz % g.batch[1], b2 = bz / g.batch[1];
-    const long long a_off = b0 * g.A.batch_stride[0] + b1 * g.A.batch_stride[1] + b2 * g.A.batch_stride[2];
-    const long long b_off = b0 * g.B.batch_stride[0] + b1 * g.B.batch_stride[1] + b2 * g.B.batch_stride[2];
-    const int       m0 = tm * FBM, n0 = tn * FBN;
-    const long long lda = (A_KC ? g.A.stride_f : g.A.stride_k) * ES; // bytes between rows of the staged A tile
-    const long long ldb = (B_KC ? g.B.stride_f : g.B.stride_k) * ES;
-    const uint8_t*  A = (const uint8_t*) g.A.base + a_off * ES;
-    const uint8_t*  B = (const uint8_t*) g.B.base + b_off * ES;
-    const uint32_t  lds_base = (uint32_t) (uintptr_t) lds;
-
-    v16f acc[4][2];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-
-    // split-k: blockIdx.z takes an equal slice of the stages and writes raw partial sums to the workspace
-    const int nk = g.K * ES / FBK / (g.split_k > 1 ? g.split_k : 1), kt_begin = (g.split_k > 1 ? (int) blockIdx.z : 0) * nk;
-    // per-lane global pointers of this wavefront's 2 + 2 request slots (they advance by one stage per step)
-    const uint8_t* ga[2];
-    const uint8_t* gb[2];
-#pragma unroll
-    for (int u = 0; u < 2; u++)
-    {
-        const int t = wave * 2 + u;
-        if constexpr (AMODE == 0)
-        {
-            const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-            ga[u] = A + (size_t) (m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
-        }
-        if constexpr (AMODE == 2)
-        {
-            const int k = t * 2 + (lane >> 5), p = lane & 31, chunk = p ^ ((k & 3) << 1);
-            ga[u] = A + (size_t) (k + kt_begin * (FBK / 2)) * lda + m0 * 2 + chunk * 16;
-        }
-        if (B_KC)
-        {
-            const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-            gb[u] = B + (size_t) (n0 + r) * ldb + c * 16 + (size_t) kt_begin * FBK;
-        }
-        else if (GATHER && g.B.kind == VIEW_TAPPED)
-            gb[u] = nullptr; // (tapped weights are k-contiguous: B_KC)
-        else if (ES == 1)
-        {
-            const int k = t * 4 + (lane >> 4), p = lane & 15, cb = (p - 2 * (k & 7)) & 15;
-            gb[u] = B + (size_t) (k + kt_begin * FBK) * ldb + n0 + cb * 16;
-        }
-        else
-        {
-            const int k = t * 2 + (lane >> 5), p = lane & 31, chunk = p ^ ((k & 3) << 1);
-            gb[u] = B + (size_t) (k + kt_begin * (FBK / 2)) * ldb + n0 * 2 + chunk * 16;
-        }
-    }
-    // ---- GATHER: per-row tap masks and the running (tap, channel) position of the stage being requested ----------------
-    uint32_t  tap_ok[2] = {0, 0};      // bit t: tap t of this lane's row (request slot u) reads inside the source tensor
-    int       g_tap = 0, g_ch = 0;     // uniform: tap and first channel of the next stage to request
-    int       g_t[3] = {0, 0, 0};      // g_tap as (s, r, q)
-    long long g_delta_a = 0, g_delta_b = 0; // uniform byte offsets of that stage: tap offset + channel
-    const int stage_ch = FBK / ES;     // channels per stage
-    auto      gather_offsets = [&]() __attribute__((always_inline))
-    {
-        long long d = 0;
-#pragma unroll
-        for (int q = 0; q < 3; q++) d += (long long) g_t[q] * g.A.dil[q] * g.A.src_stride[q];
-        g_delta_a = ((g.A.gather_y ? -d : d) + g_ch) * ES;
-        g_delta_b = ((long long) g_tap * g.B.tap_stride + g_ch) * ES;
-    };
-    auto gather_advance = [&]() __attribute__((always_inline))
-    {
-        g_ch += stage_ch;
-        if (g_ch >= g.A.nch)
-        {
-            g_ch = 0;
-            g_tap++;
-            if (++g_t[0] == g.A.ktap[0])
-            {
-                g_t[0] = 0;
-                if (++g_t[1] == g.A.ktap[1])
-                {
-                    g_t[1] = 0;
-                    g_t[2]++;
-                }
-            }
-        }
-        gather_offsets();
-    };
-    if constexpr (GATHER)
-    {
-        const int ntaps = g.A.ktap[0] * g.A.ktap[1] * g.A.ktap[2];
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-        {
-            const int r = (wave * 2 + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-            const int pix = min(m0 + r, g.M - 1);
-            const PixelPos pp = decode_pixel(g.A, pix);
-            long long      off0 = 0;
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-                off0 += (long long) (g.A.gather_y ? pp.c[d] + g.A.pad[d] : pp.c[d] * g.A.cstride[d] - g.A.pad[d]) * g.A.src_stride[d];
-            ga[u] = A + off0 * ES + c * 16;
-            if (m0 + r < g.M)
-                for (int t = 0; t < ntaps; t++) tap_ok[u] |= (conv_offset(g.A, pp, t) >= 0 ? 1u : 0u) << t;
-            if (g.B.kind == VIEW_TAPPED) gb[u] = B + (size_t) (n0 + r) * ldb + c * 16;
-        }
-        // first stage of this workgroup's k range
-        const int k0 = kt_begin * stage_ch;
-        g_tap = k0 / g.A.nch;
-        g_ch = k0 - g_tap * g.A.nch;
-        g_t[0] = g_tap % g.A.ktap[0];
-        g_t[1] = (g_tap / g.A.ktap[0]) % g.A.ktap[1];
-        g_t[2] = g_tap / (g.A.ktap[0] * g.A.ktap[1]);
-        gather_offsets();
-    }
-    // ---- AMODE 3: this lane's (tap, channel) per request slot and the pixel of the next stage to request -----------------
-    int       w_pc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}}; // pixel coordinates (dims 1..4 of the tensor that enumerates pixels)
-    int       w_t[2][3] = {{0, 0, 0}, {0, 0, 0}};        // tap as (s, r, q)
-    long long w_ch[2] = {0, 0};                          // channel byte offset, < 0: f beyond M
-    float     w_rcp[3] = {0.0f, 0.0f, 0.0f};             // 1 / grid[d]
-    if constexpr (AMODE == 3)
-    {
-#pragma unroll
-        for (int d = 0; d < 3; d++) w_rcp[d] = __builtin_amdgcn_rcpf((float) g.A.grid[d]);
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-        {
-            const int kr = (wave * 2 + u) * 2 + (lane >> 5), chunk = (lane & 31) ^ ((kr & 3) << 1);
-            const int f = m0 + chunk * 8, tap = f / g.A.nch;
-            w_ch[u] = f < g.M ? (long long) (f - tap * g.A.nch) * 2 : -1;
-            w_t[u][0] = tap % g.A.ktap[0];
-            w_t[u][1] = (tap / g.A.ktap[0]) % g.A.ktap[1];
-            w_t[u][2] = tap / (g.A.ktap[0] * g.A.ktap[1]);
-            const PixelPos pp = decode_pixel(g.A, kt_begin * (FBK / 2) + kr);
-#pragma unroll
-            for (int d = 0; d < 4; d++) w_pc[u][d] = pp.c[d];
-        }
-    }
-    auto issue_a = [&](int u, int stage, int slot) __attribute__((always_inline))
-    {
-        if constexpr (AMODE == 3)
-        {
-            // x[pos(pixel, tap)][channel .. + 7], or zeros where the tap falls into the padding
-            long long off = w_ch[u];
-            bool      ok = off >= 0;
-#pragma unroll
-            for (int d = 0; d < 4; d++)
-            {
-                const int pos = w_pc[u][d] * g.A.cstride[d] + (d < 3 ? w_t[u][d] * g.A.dil[d] : 0) - g.A.pad[d];
-                ok = ok && pos >= 0 && pos < g.A.src[d];
-                off += (long long) pos * g.A.src_stride[d] * 2;
-            }
-            const uint8_t* src = ok ? A + off : (const uint8_t*) gf_zero_page;
-            dma16(src, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
-            // next stage: 32 pixels further
-            int carry = 32;
-#pragma unroll
-            for (int d = 0; d < 3; d++)
-            {
-                // v / grid[d] for small non-negative v: float estimate, corrected by one
-                const int v = w_pc[u][d] + carry, gd = g.A.grid[d];
-                int       q = (int) ((float) v * w_rcp[d]);
-                const int r = v - q * gd;
-                q += (r >= gd) - (r < 0);
-                carry = q;
-                w_pc[u][d] = v - q * gd;
-            }
-            w_pc[u][3] += carry;
-        }
-        else if constexpr (AMODE == 2)
-            dma16(ga[u] + (size_t) stage * (FBK / ES) * lda, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
-        else if constexpr (GATHER)
-        {
-            const bool     ok = (tap_ok[u] >> g_tap) & 1u;
-            const uint8_t* src = ok ? ga[u] + g_delta_a : (const uint8_t*) gf_zero_page;
-            dma16(src, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
-        }
-        else
-            dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
-    };
-    auto issue_b = [&](int u, int stage, int slot) __attribute__((always_inline))
-    {
-        if (GATHER && g.B.kind == VIEW_TAPPED)
-        {
-            dma16(gb[u] + g_delta_b, lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
-            if (u == 1) gather_advance(); // the stage's last request
-            return;
-        }
-        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
-        if (GATHER && u == 1) gather_advance();
-    };
-    auto read_b = [&](Frags & f, int j, const char* st) __attribute__((always_inline))
-    {
-        if (B_KC) read_b_kc(f, j, st, wn, lane);
-        else if (ES == 1)
-            read_b_tr(f, j, st, wn, lane);
-        else
-            read_b_tr16(f, j, st, wn, lane);
-    };
-
-    for (int t = 0; t < FNST - 1; t++)
-    {
-#pragma unroll
-        for (int u = 0; u < 2; u++)
-        {
-            issue_a(u, t, t);
-            issue_b(u, t, t);
-        }
-    }
-    // s_waitcnt immediate (gfx9): vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-    __builtin_amdgcn_s_waitcnt(0x0F78); // vmcnt(8): stage 0 has landed
-    __syncthreads();
-    auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
-    {
-        if constexpr (A_KC) read_a(fr, i, st, wm, lane);
-        else
-            read_a_tr16(fr, i, st, wm, lane);
-    };
-    Frags f;
-#pragma unroll
-    for (int i = 0; i < 4; i++) read_a_any(f, i, lds);
-#pragma unroll
-    for (int j = 0; j < 2; j++) read_b(f, j, lds);
-
-    auto mma = [&](int i, int j) __attribute__((always_inline))
-    {
-        if constexpr (ES == 1)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
-        else
-        {
-            union
-            {
-                v8i  v;
-                v8bf h[2];
-            } ua, ub;
-            ua.v = f.a[i];
-            ub.v = f.b[j];
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ub.h[0], ua.h[0], acc[i][j], 0, 0, 0);
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ub.h[1], ua.h[1], acc[i][j], 0, 0, 0);
-        }
-    };
-#define MMA(i, j) mma(i, j)
-#define RA(i) \
-    if (RN) read_a_any(f, i, st);
-#define RB(j) \
-    if (RN) read_b(f, j, st);
-#define LA(u) \
-    if (LOADS) issue_a(u, t + FNST - 1, slot);
-#define LB(u) \
-    if (LOADS) issue_b(u, t + FNST - 1, slot);
-    // One stage: 8 MFMAs; after the first one wait until stage t+1 has landed in every wavefront's view (WAITC leaves the
-    // younger stage in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
-    // other wavefront on the SIMD covers the tail of that latency); request stage t+3.
-    auto step = [&](int t, auto waitc, auto loads, auto readnext) __attribute__((always_inline))
-    {
-        constexpr int  WAITC = decltype(waitc)::value;
-        constexpr bool LOADS = decltype(loads)::value;
-        constexpr bool RN = decltype(readnext)::value;
-        const char*    st = lds + ((t + 1) % FNST) * FSTAGE;
-        const int      slot = (t + FNST - 1) % FNST;
-        MMA(0, 0);
-        FENCE;
-        if (RN)
-        {
-            __builtin_amdgcn_s_waitcnt(WAITC);
-            __builtin_amdgcn_s_barrier();
-        }
-        FENCE;
-        MMA(0, 1); FENCE;
-        RA(0) LA(0) MMA(1, 0); FENCE;
-        MMA(1, 1); FENCE;
-        RA(1) LA(1) MMA(2, 0); FENCE;
-        MMA(2, 1); FENCE;
-        RA(2) LB(0) MMA(3, 0); FENCE;
-        RB(0) LB(1) MMA(3, 1); FENCE;
-        RA(3) RB(1) FENCE;
-    };
-    using W8 = std::integral_constant<int, 0x0F74>; // vmcnt(4): one stage of this wavefront's requests may still be in flight
-    using W0 = std::integral_constant<int, 0x0F70>; // vmcnt(0)
-    using T = std::true_type;
-    using F = std::false_type;
-    int t = 0;
-    for (; t + 5 <= nk; t += 2)
-    {
-        step(t, W8 {}, T {}, T {});
-        step(t + 1, W8 {}, T {}, T {});
-    }
-    // t == nk - 4 (nk is even and >= 6)
-    step(t, W8 {}, T {}, T {});     // requests the last stage
-    step(t + 1, W8 {}, F {}, T {}); // stage nk-2 needed, stage nk-1 may be in flight
-    step(t + 2, W0 {}, F {}, T {});
-    step(t + 3, W0 {}, F {}, F {});
-#undef MMA
-#undef RA
-#undef RB
-#undef LA
-#undef LB
-
-    // ---- epilogue: alpha, per-column power of two, relu, cast, store (same conversion functions as the general kernel).
-    // The matrix-core operands are swapped (B fragment first), so accumulator register v of lane l is output column
-    // 8 * (v / 4) + 4 * (l / 32) + v % 4 of row l % 32 of its 32 x 32 block: one v_permlane32_swap per register pair leaves
-    // every lane with 16 consecutive columns of one row, stored 16 bytes at a time.  The output-type dispatch sits
-    // outside the unrolled block walk so that the accumulators stay in registers.
-    const long long c_off = b0 * g.epi.batch_stride[0] + b1 * g.epi.batch_stride[1] + b2 * g.epi.batch_stride[2];
-    const long long ldc = g.epi.ld;
-    const bool      has_alpha = g.epi.has_alpha != 0;
-    const float     alpha = g.epi.alpha;
-    const int32_t*  col_exp = g.epi.col_exp;
-    const bool      relu = g.epi.fused && g.epi.cast.relu;
-    const int       dt = g.epi.fused ? g.epi.out_dtype : DT_FP32;
-    const int       esz = (dt == DT_FP32) ? 4 : (dt == DT_BF16 ? 2 : 1);
-    const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
-                           g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
-    const int       kg = lane >> 5;
-    // element offset of this lane's first value in block (0, 0): row m0 + wm * 128 + lane % 32, column n0 + wn * 64 + 16 kg
-    const long long lane_elem = c_off + (long long) (m0 + wm * 128 + (lane & 31)) * ldc + n0 + wn * 64 + kg * 16;
-    // block (i, j) -> the lane's 16 values after the power-of-two factors and relu
-    auto gather = [&](int i, int j, float (&val)[16]) __attribute__((always_inline))
-    {
-#pragma unroll
-        for (int q = 0; q < 2; q++)
-#pragma unroll
-            for (int r = 0; r < 4; r++)
-            {
-                const float lo = acc[i][j][4 * q + r], hi = acc[i][j][8 + 4 * q + r];
-                const auto  sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
-                val[8 * q + r] = __uint_as_float(sw[0]);
-                val[8 * q + 4 + r] = __uint_as_float(sw[1]);
-            }
-        if (has_alpha)
-        {
-#pragma unroll
-            for (int c = 0; c < 16; c++) val[c] *= alpha;
-        }
-        if (col_exp)
-        {
-#pragma unroll
-            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
-        }
-        if (relu)
-        {
-#pragma unroll
-            for (int c = 0; c < 16; c++) val[c] = relu_ref(val[c]);
-        }
-    };
-    auto walk = [&](auto store) __attribute__((always_inline))
-    {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-            {
-                float val[16];
-                gather(i, j, val);
-                if (!RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
-            }
-    };
-    typedef float    e_v4f __attribute__((ext_vector_type(4)));
-    typedef uint32_t e_v4u __attribute__((ext_vector_type(4)));
-    typedef float    e_v2f __attribute__((ext_vector_type(2)));
-    typedef __bf16   e_v2bf __attribute__((ext_vector_type(2)));
-    if (g.split_k > 1)
-    {
-        // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
-        float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N +
-                    (long long) (m0 + wm * 128 + (lane & 31)) * g.N + n0 + wn * 64 + kg * 16;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-            {
-                e_v4f*     o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
-                const bool row_ok = !RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M;
-#pragma unroll
-                for (int q = 0; q < 2; q++)
-                {
-                    float lo4[4], hi4[4];
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                    {
-                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint((float) acc[i][j][4 * q + r]),
-                                                                         __float_as_uint((float) acc[i][j][8 + 4 * q + r]), false, false);
-                        lo4[r] = __uint_as_float(sw[0]);
-                        hi4[r] = __uint_as_float(sw[1]);
-                    }
-                    if (row_ok)
-                    {
-                        o[2 * q] = e_v4f {lo4[0], lo4[1], lo4[2], lo4[3]};
-                        o[2 * q + 1] = e_v4f {hi4[0], hi4[1], hi4[2], hi4[3]};
-                    }
-                }
-            }
-    }
-    else if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
-        walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
-            e_v4f* o = (e_v4f*) ((float*) g.epi.out + idx);
-#pragma unroll
-            for (int c = 0; c < 4; c++) o[c] = e_v4f {val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3]};
-        });
-    else if (dt == DT_BF16 && g.epi.fast_cast)
-        // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN (checked over
-        // all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x| over
-        // the lane's 16 values detects them and the block is then converted element by element
-        walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
-            float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
-            const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
-            uint32_t   pk[8];
-            if (__builtin_amdgcn_ballot_w64(special) == 0)
-            {
-#pragma unroll
-                for (int c = 0; c < 8; c++)
-                {
-                    const e_v2bf h = __builtin_convertvector(e_v2f {val[2 * c], val[2 * c + 1]}, e_v2bf);
-                    __builtin_memcpy(&pk[c], &h, 4);
-                }
-            }
-            else
-            {
-#pragma unroll
-                for (int c = 0; c < 8; c++)
-                    pk[c] = fp32_to_bf16_rne(f2u(val[2 * c]), cp.clip_fp, cp.clip_inf_in) | (fp32_to_bf16_rne(f2u(val[2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
-            }
-            e_v4u* o = (e_v4u*) ((uint16_t*) g.epi.out + idx);
-            o[0] = e_v4u {pk[0], pk[1], pk[2], pk[3]};
-            o[1] = e_v4u {pk[4], pk[5], pk[6], pk[7]};
-        });
-    else if ((dt == DT_FP8_143 || dt == DT_FP8_152) && g.epi.fast_cast)
-    {
-        auto fp8_store = [&](auto m_c) __attribute__((always_inline))
-        {
-            constexpr int MAN = decltype(m_c)::value;
-            walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
-                // the hardware converter equals the reference's conversion on finite inputs; a block that holds inf or
-                // NaN (sum of magnitudes not finite) takes the exact converter
-                float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
-                const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) <= 0x1.fffffep+127f);
-                uint32_t   pk[4];
-                if (__builtin_amdgcn_ballot_w64(special) == 0)
-                {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) pk[c] = fp8_hw_pack4<MAN>(val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3], cp.exp_bias, cp.clip_fp);
-                }
-                else
-                {
-#pragma unroll
-                    for (int c = 0; c < 4; c++)
-                    {
-                        pk[c] = 0;
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            pk[c] |= (fp32_to_fp8_rne_mode0<MAN>(f2u(val[4 * c + e]), cp.exp_bias, cp.clip_fp, cp.clip_inf_in) & 0xFFu) << (8 * e);
-                    }
-                }
-                *(e_v4u*) ((uint8_t*) g.epi.out + idx) = e_v4u {pk[0], pk[1], pk[2], pk[3]};
-            });
-        };
-        if (dt == DT_FP8_143) fp8_store(std::integral_constant<int, 3>());
-        else
-            fp8_store(std::integral_constant<int, 2>());
-    }
-    else
-    {
-        // rare cast settings: element-wise through the out-of-line generic converter (which applies relu itself)
-#pragma unroll 1
-        for (int i = 0; i < 4; i++)
-#pragma unroll 1
-            for (int j = 0; j < 2; j++)
-            {
-                float val[16];
-#pragma unroll
-                for (int q = 0; q < 2; q++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                    {
-                        // (dynamic block index: read the accumulators through a switch-free copy)
-                        float lo = 0.0f, hi = 0.0f;
-#pragma unroll
-                        for (int ii = 0; ii < 4; ii++)
-#pragma unroll
-                            for (int jj = 0; jj < 2; jj++)
-                                if (ii == i && jj == j)
-                                {
-                                    lo = acc[ii][jj][4 * q + r];
-                                    hi = acc[ii][jj][8 + 4 * q + r];
-                                }
-                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
-                        val[8 * q + r] = __uint_as_float(sw[0]);
-                        val[8 * q + 4 + r] = __uint_as_float(sw[1]);
-                    }
-                for (int c = 0; c < 16; c++)
-                {
-                    float x = val[c];
-                    if (has_alpha) x *= alpha;
-                    if (col_exp) x *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
-                    if (!RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
-                }
-            }
-    }
-    (void) esz;
-}
-
 template<int FMT, bool B_KC>
 __global__ __launch_bounds__(512) void gemm_fp8_fast_kernel(GemmProblem g_by_value)
 {
@@ -723,19 +80,6 @@ hipError_t launch_conv_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
     return hipGetLastError();
 }
 
-template<class K>
-hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s)
-{
-    if (!attr_done)
-    {
-        hipError_t e = hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FNST * FSTAGE);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
-    hipLaunchKernelGGL(kernel, grid, dim3(512), FNST * FSTAGE, s, p);
-    return hipGetLastError();
-}
-
 hipError_t launch_bf16(const GemmProblem& p, dim3 grid, hipStream_t s)
 {
     static bool attr_done[5] = {false, false, false, false, false};
@@ -766,15 +110,18 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 }
 } // namespace
 
+hipError_t launch_gemm_large_tile_f16(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_f16.hip
+
 bool gemm_large_tile_applicable(const GemmProblem& p)
 {
-    if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152 || p.dtype == DT_BF16)) return false;
-    const int es = p.dtype == DT_BF16 ? 2 : 1;
+    if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152 || p.dtype == DT_BF16 || p.dtype == DT_FP16)) return false;
+    const bool two_byte = p.dtype == DT_BF16 || p.dtype == DT_FP16;
+    const int  es = two_byte ? 2 : 1;
     const bool gather = p.A.kind == VIEW_CONV;
     if (gather)
     {
-        // bf16, at most 32 taps, one problem per launch
-        if (p.dtype != DT_BF16 || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
+        // bf16 / fp16, at most 32 taps, one problem per launch
+        if (!two_byte || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
         if (p.batch[0] * p.batch[1] * p.batch[2] != 1) return false;
         if (p.A.pix_is_f)
         {
@@ -795,7 +142,7 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     else if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN)
         return false;
     if (!p.A.vec_ok || !p.B.vec_ok) return false;
-    if (!p.A.k_contig && p.dtype != DT_BF16) return false; // f-contiguous A: bf16 only
+    if (!p.A.k_contig && !two_byte) return false; // f-contiguous A: bf16 / fp16 only
     if (gather && p.A.pix_is_f && !p.A.k_contig) return false;
     if ((!gather && p.M % FBM) || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
     if (p.split_k > 1)
@@ -823,7 +170,7 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
     q.split_k = 1;
     if (!gemm_large_tile_applicable(q)) return 0;
     const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
-    const int       nk = p.K * (p.dtype == DT_BF16 ? 2 : 1) / FBK;
+    const int       nk = p.K * dt_bytes(p.dtype) / FBK;
     int             best = 1;
     // Splitting the reduction pays when the tiles leave most of the chip idle and the reduction is long: a slice costs a
     // pass of the fp32 output through the workspace plus the reduction kernel.  Rough model in microseconds: a stage (128 bytes of
@@ -850,6 +197,7 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     dim3            grid(((p.M + FBM - 1) / FBM) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return launch_conv_bf16(p, grid, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))

@@ -800,9 +800,18 @@ int mme_hip_activation_dev(mme_hip_handle h, const mme_hip_tensor* out, const mm
     if (!(out->dtype == MME_HIP_FP32 || out->dtype == MME_HIP_BF16 || is_fp8(out->dtype) || is_fp16(out->dtype)))
         return fail(h, MME_HIP_EINVAL, "Unsupported type");
     if (!(rm == 0 || rm == 1 || rm == 2 || rm == 3 || rm == 4 || rm == 6 || rm == 7)) return fail(h, MME_HIP_EINVAL, "invalid rounding mode %d", rm);
-    // the reference converts the first getSizeInElements() elements of both flat buffers (:1155)
-    const size_t n = n_elements(acc);
-    if (relu) HIP_TRY(h, launch_relu_inplace((float*) acc->data, n, h->stream));
+    // the reference converts the first getSizeInElements() elements of both flat buffers (:1155), and that count is the
+    // tensor's span in memory, gaps between strided rows included (sim_tensor_base.cpp:177-194)
+    const size_t n = span_elements(acc);
+    if (span_elements(out) < n) return fail(h, MME_HIP_EINVAL, "the output tensor spans fewer elements than acc");
+    if (relu)
+    {
+        // doRelu insists on a tensor without gaps (mme_reference_impl.cpp:1135)
+        bool contiguous = acc->strides[0] == 1;
+        for (int d = 1; d < acc->dim && d < MME_HIP_MAX_TENSOR_DIMS; d++) contiguous = contiguous && acc->strides[d] == acc->strides[d - 1] * acc->sizes[d - 1];
+        if (!contiguous) return fail(h, MME_HIP_EINVAL, "input and output should be flattened");
+        HIP_TRY(h, launch_relu_inplace((float*) acc->data, n, h->stream));
+    }
     const CastParams c = make_cast(out->dtype, out->fp_bias, out->inf_nan_mode, rm, clip_fp, clip_inf_in, flush_denorms, 0, 0);
     const bool       reseed = rm == MME_HIP_RM_STOCHASTIC || rm == MME_HIP_RM_STOCHASTIC_AND_NEAREST || stochastic_ftz;
     if (reseed && out->dtype != MME_HIP_FP32)

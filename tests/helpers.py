@@ -47,6 +47,11 @@ def random_operand(rng, dtype, n, orc=None, bias=7, mode=0, scale=1.0):
         return to_bf16_bits(x)
     if dtype == abi.FP32:
         return x
+    if dtype in (abi.FP16, abi.UFP16):
+        out = np.zeros(n, np.uint16)
+        src = np.abs(x) if dtype == abi.UFP16 else x
+        assert orc.orc_cast_from_fp32(out.ctypes.data, dtype, bias, mode, src.ctypes.data, n, 0, None, 0, 0, 0, 1, 0, 0) == 0
+        return out
     return quantize_fp8(orc, x, dtype, bias, mode)
 
 

@@ -222,3 +222,30 @@ def test_memory_write_reductions(calc, orc, dt):
     calc.doMemoryWrite(MmeSimTensor(sizes, 5, dt, tm), MmeSimTensor(sizes, 5, dt, tb))
     calc.synchronize()
     assert np.array_equal(tm.cpu().numpy().view(a.dtype), b)
+
+
+@pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP8_143, 7), (abi.FP16, 15), (abi.FP32, 0)])
+def test_activation_converts_the_whole_span_of_strided_tensors(calc, orc, dt, bias):
+    """A strided output: the reference's doActivation converts every flat element of the tensor's span, the gaps between
+    rows included; device and host tensors against the oracle, bit for bit.  relu on such a tensor is refused like the
+    reference refuses it."""
+    import torch
+    from intel_gaudi3_software_amd import MMEStackException, MmeSimTensor
+    rng = np.random.default_rng(26)
+    sizes, strides = [5, 4, 3, 1, 1], [1, 7, 30, 90, 90]
+    acc = rng.standard_normal(90).astype(np.float32)
+    want = np.full(90, 0x11, abi.DTYPE_NUMPY[dt])
+    a_ref = acc.copy()
+    d_o, d_a = desc(want, sizes, dt, bias, 0, strides), desc(a_ref, sizes, abi.FP32, 0, 0, strides)
+    assert orc.orc_activation(A(d_o), A(d_a), 0, 0, 1, 0, 0, 0, None, 0) == 0
+    host_out, host_acc = np.full(90, 0x11, abi.DTYPE_NUMPY[dt]), acc.copy()
+    calc.doActivation(MmeSimTensor(sizes, 5, dt, host_out, bias, 0, strides), MmeSimTensor(sizes, 5, abi.FP32, host_acc, strides=strides), clipFp=True)
+    assert np.array_equal(host_out.view(np.uint8), want.view(np.uint8))
+    view = {1: np.uint8, 2: np.int16, 4: np.float32}[abi.DTYPE_SIZE[dt]]
+    o_d = torch.from_numpy(np.full(90, 0x11, abi.DTYPE_NUMPY[dt]).view(view).copy()).cuda()
+    a_d = torch.from_numpy(acc.copy()).cuda()
+    calc.doActivation(MmeSimTensor(sizes, 5, dt, o_d, bias, 0, strides), MmeSimTensor(sizes, 5, abi.FP32, a_d, strides=strides), clipFp=True)
+    calc.synchronize()
+    assert np.array_equal(o_d.cpu().numpy().view(np.uint8), want.view(np.uint8))
+    with pytest.raises(MMEStackException, match="should be flattened"):
+        calc.doActivation(MmeSimTensor(sizes, 5, dt, o_d, bias, 0, strides), MmeSimTensor(sizes, 5, abi.FP32, a_d, strides=strides), relu=True)

@@ -307,3 +307,35 @@ def test_tf32_rounding_is_applied_before_the_products(calc, orc):
     got, want = _gemm_both(calc, orc, abi.OP_ABT, M, N, K, PAIRS[6], a.view(np.uint32), b.view(np.uint32))
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     assert np.all(want == np.round(want)) and np.any(want != 0)
+
+
+@pytest.mark.parametrize("op", OPS)
+@pytest.mark.parametrize("pair", PAIRS[:2])
+def test_fp16_large_tile_kernel(calc, orc, op, pair):
+    """fp16 shapes that take the large-tile kernel (M, N multiples of 256, K a multiple of 64 and at least 192), all four
+    layouts, a batch of two with B broadcast; and a long reduction over few tiles, which is split over k."""
+    rng = np.random.default_rng(200 + op)
+    for (M, N, K, batch) in [(256, 512, 320, (2, 1, 1)), (256, 256, 4096, (1, 1, 1))]:
+        nb = int(np.prod(batch))
+        a = _operand(rng, orc, pair[0], pair[2], pair[4], M * K * nb)
+        b = _operand(rng, orc, pair[1], pair[3], pair[5], N * K)
+        got, want = _gemm_both(calc, orc, op, M, N, K, pair, a, b, batch)
+        assert rel_frobenius(got, want) <= 1e-4, (M, N, K)
+
+
+def test_fp16_large_tile_every_k_position(calc, orc):
+    """One-hot fp16 operands walk a single product through every k position and tile coordinate of the large-tile kernel."""
+    M, N, K = 256, 256, 384
+    a = np.zeros((M, K), np.float32)
+    b = np.zeros((K, N), np.float32)
+    rng = np.random.default_rng(5)
+    perm_m = rng.permutation(M)
+    for k in range(K):
+        a[perm_m[k % M], k] = 1.0 + (k % 5)
+        b[k, (k * 11 + 2) % N] = 2.0 if k % 2 else 1.0
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    for b_kc in (False, True):
+        bmat = b.T.copy() if b_kc else b
+        ha, hb = a.astype(np.float16).view(np.uint16).ravel(), bmat.astype(np.float16).view(np.uint16).ravel()
+        got, ref = _gemm_both(calc, orc, abi.OP_ABT if b_kc else abi.OP_AB, M, N, K, PAIRS[0], ha, hb)
+        assert np.array_equal(got.reshape(M, N), want) and np.array_equal(ref.reshape(M, N), want)
