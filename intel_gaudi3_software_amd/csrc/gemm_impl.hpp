@@ -336,9 +336,10 @@ __device__ __forceinline__ void mma_slab(v16f& acc, const Slab& a, const Slab& b
 // ------------------------------------------------------------------------------------------------------------
 // fp16 / ufp16 outputs: one out-of-line copy of the converter, so that the unrolled epilogues of the other output types
 // keep their size
-__device__ __attribute__((noinline)) uint32_t cast_half_out_of_line(float v, const CastParams& cp)
+__device__ __attribute__((noinline)) uint32_t cast_half_out_of_line(float v, const CastParams& cp, int fast)
 {
-    return cp.dtype == DT_UFP16 ? cast_elem<DT_UFP16, false>(v, cp) : cast_elem<DT_FP16, false>(v, cp);
+    if (cp.dtype == DT_UFP16) return cast_elem<DT_UFP16, false>(v, cp);
+    return fast ? cast_elem<DT_FP16, true>(v, cp) : cast_elem<DT_FP16, false>(v, cp);
 }
 
 __device__ __forceinline__ void store_out(EpilogueRef e, long long idx, float v)
@@ -362,7 +363,7 @@ __device__ __forceinline__ void store_out(EpilogueRef e, long long idx, float v)
             ((uint16_t*) e.out)[idx] = (uint16_t) (e.fast_cast ? cast_elem<DT_BF16, true>(v, cp) : cast_elem<DT_BF16, false>(v, cp));
             break;
         case DT_FP16:
-        case DT_UFP16: ((uint16_t*) e.out)[idx] = (uint16_t) cast_half_out_of_line(v, cp); break;
+        case DT_UFP16: ((uint16_t*) e.out)[idx] = (uint16_t) cast_half_out_of_line(v, cp, e.fast_cast); break;
         default: ((uint32_t*) e.out)[idx] = cast_elem<DT_FP32, false>(v, cp); break;
     }
 }
