@@ -578,6 +578,8 @@ __global__ __launch_bounds__(CAST_THREADS) void memory_write_reduce_kernel(void*
             for (int w = 0; w < 4; w++)
             {
                 if constexpr (DT == DT_FP32) r[w] = rmw_elem<23>(a[w], b[w], op, rm, clip);
+                else if constexpr (DT == DT_FP16)
+                    r[w] = rmw_elem_fp16(a[w] & 0xFFFFu, b[w] & 0xFFFFu, op, rm, clip) | (rmw_elem_fp16(a[w] >> 16, b[w] >> 16, op, rm, clip) << 16);
                 else
                     r[w] = (rmw_elem<7>(a[w] << 16, b[w] << 16, op, rm, clip) >> 16) |
                            (rmw_elem<7>(a[w] & 0xFFFF0000u, b[w] & 0xFFFF0000u, op, rm, clip) & 0xFFFF0000u);
@@ -589,6 +591,8 @@ __global__ __launch_bounds__(CAST_THREADS) void memory_write_reduce_kernel(void*
     for (size_t i = done + t; i < n; i += stride)
     {
         if constexpr (DT == DT_FP32) ((uint32_t*) memory)[i] = rmw_elem<23>(((uint32_t*) memory)[i], ((const uint32_t*) mme_out)[i], op, rm, clip);
+        else if constexpr (DT == DT_FP16)
+            ((uint16_t*) memory)[i] = (uint16_t) rmw_elem_fp16(((uint16_t*) memory)[i], ((const uint16_t*) mme_out)[i], op, rm, clip);
         else
             ((uint16_t*) memory)[i] =
                 (uint16_t) (rmw_elem<7>((uint32_t) ((uint16_t*) memory)[i] << 16, (uint32_t) ((const uint16_t*) mme_out)[i] << 16, op, rm, clip) >> 16);
@@ -603,6 +607,8 @@ hipError_t launch_memory_write_reduce(void* memory, const void* mme_out, int dty
     if (dtype == DT_FP32) hipLaunchKernelGGL(memory_write_reduce_kernel<DT_FP32>, grid, block, 0, s, memory, mme_out, n, op, rm, clip, vec_ok);
     else if (dtype == DT_BF16)
         hipLaunchKernelGGL(memory_write_reduce_kernel<DT_BF16>, grid, block, 0, s, memory, mme_out, n, op, rm, clip, vec_ok);
+    else if (dtype == DT_FP16)
+        hipLaunchKernelGGL(memory_write_reduce_kernel<DT_FP16>, grid, block, 0, s, memory, mme_out, n, op, rm, clip, vec_ok);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();

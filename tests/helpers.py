@@ -117,6 +117,28 @@ def rmw_operands(rng, dt, n):
     return a, b
 
 
+def rmw_operands_fp16(rng, n):
+    """The same families for fp16 (5 exponent bits, 10 mantissa bits)."""
+    rand = lambda k: rng.integers(0, 1 << 16, k, dtype=np.uint64).astype(np.uint16)
+    a, b = rand(n), rand(n)
+    q = n // 8
+    b[:q] = (a[:q] ^ 0x8000) ^ rng.integers(0, 4, q).astype(np.uint16)
+    ea = rng.integers(14, 31, q)
+    gap = rng.integers(8, 15, q)
+    sgn = rng.integers(0, 2, (2, q))
+    a[q:2 * q] = ((sgn[0] << 15) | (ea << 10) | rng.integers(0, 1 << 10, q)).astype(np.uint16)
+    b[q:2 * q] = ((sgn[1] << 15) | ((ea - gap) << 10) | rng.integers(0, 1 << 10, q)).astype(np.uint16)
+    a[2 * q:3 * q] = ((sgn[0] << 15) | (rng.integers(0, 4, q) << 10) | rng.integers(0, 1 << 10, q)).astype(np.uint16)
+    b[2 * q:3 * q] = ((sgn[1] << 15) | (rng.integers(0, 4, q) << 10) | rng.integers(0, 1 << 10, q)).astype(np.uint16)
+    a[3 * q:4 * q] = ((sgn[0] << 15) | (rng.integers(28, 32, q) << 10) | rng.integers(0, 1 << 10, q)).astype(np.uint16)
+    b[3 * q:4 * q] = ((sgn[1] << 15) | (rng.integers(28, 32, q) << 10) | rng.integers(0, 1 << 10, q)).astype(np.uint16)
+    specials = np.array([0, 0x8000, 0x7C00, 0xFC00, 0x7C01, 1, 0x0400, 0x7BFF, 0x03FF, 0x8001, 0xFBFF, 0x3C00], np.uint16)
+    k = len(specials)
+    a[4 * q:4 * q + k * k] = np.repeat(specials, k)
+    b[4 * q:4 * q + k * k] = np.tile(specials, k)
+    return a, b
+
+
 class OracleCalculator:
     """The oracle behind CPUCalculator's method names, on host MmeSimTensor objects: lets the harness sequence
     (intel_gaudi3_software_amd.harness.run_reference_sequence) run on the CPU checker for comparison."""
