@@ -634,15 +634,11 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
         return fail(h, MME_HIP_EINVAL, "convolution extents exceed 2^31");
     if (n_elements(out) == 0) return MME_HIP_OK;
 
-    // dense weight tensor and row-collapsible outputs keep the addressing linear
-    {
-        uint64_t acc = 1;
-        for (int d = 0; d < 5; d++)
-        {
-            if (wt->sizes[d] > 1 && wt->strides[d] != acc) return fail(h, MME_HIP_EUNSUPPORTED, "strided weight tensors are not built in this library");
-            acc *= wt->sizes[d];
-        }
-    }
+    // weights with one row pitch (rows of K output channels, one per (channel, tap)) and row-collapsible outputs keep the
+    // addressing linear
+    if (!rows_collapsible(wt)) return fail(h, MME_HIP_EUNSUPPORTED, "weight tensors whose rows do not share one pitch are not built in this library");
+    const long long w_ld = (long long) taps * C > 1 ? (long long) wt->strides[1] : Kc;
+    if (w_ld < Kc) return fail(h, MME_HIP_EINVAL, "weight rows overlap");
     if (!rows_collapsible(out)) return fail(h, MME_HIP_EUNSUPPORTED, "output tensors with non-collapsible row strides are not built");
     if (op == MME_HIP_OP_DEDW && !rows_collapsible(y)) return fail(h, MME_HIP_EUNSUPPORTED, "dedw needs a row-collapsible dy tensor");
 
@@ -712,7 +708,7 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
         g.N = Kc;
         g.K = taps * C;
         conv_view(g.A, x, out, C, 1, 0);
-        set_plain_view(g.B, w->data, 1, Kc, false, es, Kc, zero3);
+        set_plain_view(g.B, w->data, 1, w_ld, false, es, Kc, zero3);
     }
     else if (op == MME_HIP_OP_DEDX)
     {
@@ -725,11 +721,11 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
         g.B.base = (const char*) w->data;
         g.B.kind = VIEW_TAPPED;
         g.B.k_contig = 1;
-        g.B.stride_f = Kc;
+        g.B.stride_f = w_ld;
         g.B.stride_k = 1;
-        g.B.tap_stride = (long long) Kc * C;
+        g.B.tap_stride = w_ld * C;
         g.B.nch = Kc;
-        g.B.vec_ok = ((uintptr_t) w->data % 16 == 0) && (Kc % kv == 0);
+        g.B.vec_ok = ((uintptr_t) w->data % 16 == 0) && (Kc % kv == 0) && (w_ld % kv == 0);
     }
     else
     {
