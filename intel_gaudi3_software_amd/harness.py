@@ -130,6 +130,9 @@ def _interpret(raw, rng):
         strides = raw.get(name + "Strides")
         t[key + "_strides"] = [_int(s) for s in strides] if strides and any(_int(s) for s in strides) else None
         t[key + "_range"] = (float(raw[name + "MinVal"]), float(raw[name + "MaxVal"]), float(raw[name + "Mean"]), float(raw[name + "Std"]))
+        sizes2, strides2 = raw.get(name + "Sizes2"), raw.get(name + "Strides2")
+        t[key + "_sizes2"] = [_int(s) for s in sizes2] if sizes2 and "random" not in sizes2 else None
+        t[key + "_strides2"] = [_int(s) for s in strides2] if strides2 and any(_int(s) for s in strides2) else None
     t["padding"] = [_int(v) for v in raw.get("padding", ("0", "0", "0"))]
     t["conv_strides"] = [_int(v) for v in raw.get("strides", ("1", "1", "1"))]
     t["dilation"] = [_int(v) for v in raw.get("dilation", ("1", "1", "1"))]
@@ -144,8 +147,8 @@ def supported(t):
         return "skipTest"
     if t["operation"] is None:
         return "operation %s is not a contraction of the calculator" % t["operation_name"]
-    if t["dual_gemm"] or t["masked_bgemm"]:
-        return "dual / masked GEMM"
+    if t["masked_bgemm"]:
+        return "masked GEMM"
     if t["out_type"] == abi.TF32:
         return "tf32 is an operand type only"
     if any(t[k + "_sizes"] is None for k in ("x", "w", "y")):
@@ -189,6 +192,21 @@ def compare_with_reference(t, device_output, reference_output, test_counter=0, p
     out_dtype, out_bias, out_mode = tensor_types(t)[o_l]
     cmp = TensorComparator(cd_size(t), out_dtype, out_bias, out_mode, print_all_diffs)
     return cmp.doCompare(device_output, "first output of Device[0]", reference_output, "Reference", test_counter, t["name"])
+
+
+def gemms_of(t):
+    """The contractions a test asks of the calculator: one, or the two of a dual-GEMM test (the test manager runs the
+    reference sequence once per gemm of the test, mme_test_manager.cpp:798-905; the second takes its sizes from the keys
+    that end in 2)."""
+    if not t["dual_gemm"]:
+        return [t]
+    second = dict(t)
+    for k in ("x", "w", "y"):
+        second[k + "_sizes"], second[k + "_strides"] = t[k + "_sizes2"], t[k + "_strides2"]
+    first = dict(t)
+    first["dual_gemm"] = second["dual_gemm"] = False
+    first["name"], second["name"] = t["name"] + " gemm 0", t["name"] + " gemm 1"
+    return [first, second]
 
 
 def operand_roles(t):

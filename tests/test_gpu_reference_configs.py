@@ -28,14 +28,17 @@ def _key(t):
 def _collect(large=False):
     cases, seen = [], set()
     for path in sorted(glob.glob(os.path.join(CONFIG_DIR, "*", "*.json"))):
-        for i, t in enumerate(harness.load_tests(path, seed=7)):
-            if harness.supported(t) is not None or (harness.contraction_flops(t) > MAX_FLOPS) != large:
+        for i, test in enumerate(harness.load_tests(path, seed=7)):
+            if harness.supported(test) is not None:
                 continue
-            k = _key(t)
-            if k in seen:  # tests that differ only in descriptor-generation parameters are one case for the calculator
-                continue
-            seen.add(k)
-            cases.append(pytest.param(t, id="%s-%d-%s" % (os.path.basename(path)[:-5], i, t["operation_name"])))
+            for g, t in enumerate(harness.gemms_of(test)):  # (a dual-GEMM test is two contractions)
+                if (harness.contraction_flops(t) > MAX_FLOPS) != large:
+                    continue
+                k = _key(t)
+                if k in seen:  # tests that differ only in descriptor-generation parameters are one case for the calculator
+                    continue
+                seen.add(k)
+                cases.append(pytest.param(t, id="%s-%d%s-%s" % (os.path.basename(path)[:-5], i, ".%d" % g if test["dual_gemm"] else "", t["operation_name"])))
     return cases
 
 

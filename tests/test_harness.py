@@ -41,3 +41,13 @@ def test_operand_roles_follow_the_operation():
     assert harness.operand_roles(tests[0]) == ("y", "w", "x")
     tests = harness.load_tests(os.path.join(CONFIG_DIR, "basic_tests", "basic_dedw.json"))
     assert harness.operand_roles(tests[0]) == ("x", "y", "w")
+
+
+def test_dual_gemm_tests_are_two_contractions():
+    tests = harness.load_tests(os.path.join(CONFIG_DIR, "basic_tests", "basic_dual_gemm.json"))
+    assert len(tests) == 7 and all(t["dual_gemm"] and harness.supported(t) is None for t in tests)
+    first, second = harness.gemms_of(tests[0])
+    assert (first["x_sizes"], first["w_sizes"], first["y_sizes"]) == ([120, 112], [80, 120], [80, 112])
+    assert (second["x_sizes"], second["w_sizes"], second["y_sizes"]) == ([128, 88], [90, 128], [90, 88])
+    assert harness.cd_size(first) == 120 and harness.cd_size(second) == 128
+    assert harness.gemms_of(first) == [first]
