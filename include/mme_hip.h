@@ -305,10 +305,12 @@ int mme_hip_activation(mme_hip_handle        h,
  * CPUCalculator::doMemoryWrite(memory, mmeOut, reductionOp, reductionRm, clipFp)
  * mme_reference.h:174-178, mme_reference_impl.cpp:718-768.  reduction_none is a
  * byte copy of memory's size.  add / sub / min / max / max_0 combine memory with
- * mmeOut element by element as the reference's executeOp does for bf16 and fp32
- * tensors (fs_fma.cpp:2288-2955: an adder that rounds once in reduction_rm and
- * flushes denormal operands and results); fp8_152 and fp16 reductions return
- * EUNSUPPORTED, the types the reference rejects return EINVAL.
+ * mmeOut element by element as the reference's executeOp does for fp32, bf16,
+ * fp16 and fp8_152 tensors (fs_fma.cpp:2288-2955: an adder that rounds once in
+ * reduction_rm and flushes denormal operands and results; fp16 and fp8_152 are
+ * taken with exponent bias 15 and inf / NaN whatever the tensor's fields say,
+ * fp8_152 sums are formed in fp16 and rounded a second time); the types the
+ * reference rejects (fp8_143, ufp16) return EINVAL.
  */
 int mme_hip_memory_write(mme_hip_handle        h,
                          const mme_hip_tensor* memory,

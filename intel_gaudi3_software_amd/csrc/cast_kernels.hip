@@ -563,7 +563,7 @@ __global__ __launch_bounds__(CAST_THREADS) void memory_write_reduce_kernel(void*
 {
     const size_t stride = (size_t) gridDim.x * CAST_THREADS;
     const size_t t = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x;
-    constexpr int PER = DT == DT_FP32 ? 4 : 8; // elements per 16 bytes
+    constexpr int PER = 16 / dt_bytes(DT); // elements per 16 bytes
     size_t        done = 0;
     if (vec_ok)
     {
@@ -580,6 +580,12 @@ __global__ __launch_bounds__(CAST_THREADS) void memory_write_reduce_kernel(void*
                 if constexpr (DT == DT_FP32) r[w] = rmw_elem<23>(a[w], b[w], op, rm, clip);
                 else if constexpr (DT == DT_FP16)
                     r[w] = rmw_elem_fp16(a[w] & 0xFFFFu, b[w] & 0xFFFFu, op, rm, clip) | (rmw_elem_fp16(a[w] >> 16, b[w] >> 16, op, rm, clip) << 16);
+                else if constexpr (DT == DT_FP8_152)
+                {
+                    r[w] = 0u;
+#pragma unroll
+                    for (int k = 0; k < 4; k++) r[w] |= rmw_elem_fp8_152((a[w] >> (8 * k)) & 0xFFu, (b[w] >> (8 * k)) & 0xFFu, op, rm, clip) << (8 * k);
+                }
                 else
                     r[w] = (rmw_elem<7>(a[w] << 16, b[w] << 16, op, rm, clip) >> 16) |
                            (rmw_elem<7>(a[w] & 0xFFFF0000u, b[w] & 0xFFFF0000u, op, rm, clip) & 0xFFFF0000u);
@@ -593,6 +599,8 @@ __global__ __launch_bounds__(CAST_THREADS) void memory_write_reduce_kernel(void*
         if constexpr (DT == DT_FP32) ((uint32_t*) memory)[i] = rmw_elem<23>(((uint32_t*) memory)[i], ((const uint32_t*) mme_out)[i], op, rm, clip);
         else if constexpr (DT == DT_FP16)
             ((uint16_t*) memory)[i] = (uint16_t) rmw_elem_fp16(((uint16_t*) memory)[i], ((const uint16_t*) mme_out)[i], op, rm, clip);
+        else if constexpr (DT == DT_FP8_152)
+            ((uint8_t*) memory)[i] = (uint8_t) rmw_elem_fp8_152(((uint8_t*) memory)[i], ((const uint8_t*) mme_out)[i], op, rm, clip);
         else
             ((uint16_t*) memory)[i] =
                 (uint16_t) (rmw_elem<7>((uint32_t) ((uint16_t*) memory)[i] << 16, (uint32_t) ((const uint16_t*) mme_out)[i] << 16, op, rm, clip) >> 16);
@@ -609,6 +617,8 @@ hipError_t launch_memory_write_reduce(void* memory, const void* mme_out, int dty
         hipLaunchKernelGGL(memory_write_reduce_kernel<DT_BF16>, grid, block, 0, s, memory, mme_out, n, op, rm, clip, vec_ok);
     else if (dtype == DT_FP16)
         hipLaunchKernelGGL(memory_write_reduce_kernel<DT_FP16>, grid, block, 0, s, memory, mme_out, n, op, rm, clip, vec_ok);
+    else if (dtype == DT_FP8_152)
+        hipLaunchKernelGGL(memory_write_reduce_kernel<DT_FP8_152>, grid, block, 0, s, memory, mme_out, n, op, rm, clip, vec_ok);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();

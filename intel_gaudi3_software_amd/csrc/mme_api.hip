@@ -997,11 +997,11 @@ int mme_hip_memory_write_dev(mme_hip_handle h, const mme_hip_tensor* memory, con
     switch (memory->dtype)
     {
         case MME_HIP_BF16:
-        case MME_HIP_FP16: // (the unit's fp16: exponent bias 15 with inf and NaN, whatever the tensor's fields say)
+        case MME_HIP_FP16:    // (the unit's fp16 and fp8_152: exponent bias 15 with inf and NaN, whatever the tensor's fields say)
+        case MME_HIP_FP8_152:
         case MME_HIP_FP32: break;
         case MME_HIP_FP8_143: return fail(h, MME_HIP_EINVAL, "fp8_143 is not supported in reduction");
         case MME_HIP_UFP16: return fail(h, MME_HIP_EINVAL, "ufp16 is not supported in reduction");
-        case MME_HIP_FP8_152: return fail(h, MME_HIP_EUNSUPPORTED, "fp8_152 reductions are not built in this library");
         default: return fail(h, MME_HIP_EINVAL, "Unsupported data type when converting to reduction RMW data type");
     }
     if (mme_out->dtype != memory->dtype) return fail(h, MME_HIP_EINVAL, "element types of memory and mmeOut differ");

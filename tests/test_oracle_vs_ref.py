@@ -205,20 +205,26 @@ def test_memory_write_reductions(orc):
     rng = np.random.default_rng(21)
     n = (1 << 18) + 1
     from helpers import rmw_operands_fp16
-    type_code = {abi.FP32: rmw.ref_rmw_type_fp32(), abi.BF16: rmw.ref_rmw_type_bf16(), abi.FP16: rmw.ref_rmw_type_fp16()}
-    for dt in (abi.FP32, abi.BF16, abi.FP16):
-        a, b = rmw_operands_fp16(rng, n) if dt == abi.FP16 else rmw_operands(rng, dt, n)
+    type_code = {abi.FP32: rmw.ref_rmw_type_fp32(), abi.BF16: rmw.ref_rmw_type_bf16(), abi.FP16: rmw.ref_rmw_type_fp16(),
+                 abi.FP8_152: rmw.ref_rmw_type_fp8()}
+    all_pairs = np.arange(65536, dtype=np.uint32)
+    for dt in (abi.FP32, abi.BF16, abi.FP16, abi.FP8_152):
+        if dt == abi.FP8_152:  # every pair of codes (plus one element: the 4-byte loop's tail)
+            a, b = np.append(all_pairs >> 8, 0x3C).astype(np.uint8), np.append(all_pairs & 0xFF, 0xBC).astype(np.uint8)
+        else:
+            a, b = rmw_operands_fp16(rng, n) if dt == abi.FP16 else rmw_operands(rng, dt, n)
         for op, rm, clip in itertools.product(range(5), range(4), (0, 1)):
             if op in (abi.REDUCTION_MIN, abi.REDUCTION_MAX) and (rm or clip):
                 continue
             m1, m2 = a.copy(), a.copy()
-            sizes = [n, 1, 1, 1, 1]
-            d2, do = desc(m2, sizes, dt, 15 if dt == abi.FP16 else 0), desc(b, sizes, dt, 15 if dt == abi.FP16 else 0)
+            sizes = [a.size, 1, 1, 1, 1]
+            d2, do = desc(m2, sizes, dt, 15 if dt in (abi.FP16, abi.FP8_152) else 0), desc(b, sizes, dt, 15 if dt in (abi.FP16, abi.FP8_152) else 0)
             rmw.ref_memory_write_words(m1.ctypes.data, b.ctypes.data, m1.nbytes, op, type_code[dt], rm, clip)
             assert orc.orc_memory_write(A(d2), A(do), op, rm, clip) == 0
             bad = np.flatnonzero(m1 != m2)
             assert bad.size == 0, (dt, op, rm, clip, hex(int(a[bad[0]])), hex(int(b[bad[0]])), hex(int(m1[bad[0]])), hex(int(m2[bad[0]])))
     # reduction none: a byte copy
+    a, b = rmw_operands(rng, abi.BF16, n)
     m1 = a.copy()
     d1, do = desc(m1, [n, 1, 1, 1, 1], abi.BF16), desc(b, [n, 1, 1, 1, 1], abi.BF16)
     assert orc.orc_memory_write(A(d1), A(do), abi.REDUCTION_NONE, 0, 0) == 0
