@@ -10,7 +10,7 @@
 //               wavefront cannot issue anything while its own MFMA occupies it, so its neighbour's MFMAs are what
 //               cover its LDS reads, DMA requests and waits
 //   HBM/L2->LDS global_load_lds_dwordx4: 16 bytes per lane straight into LDS, no staging registers.  Ring of 4 stages of
-//               64 k-bytes (A 256 x 64 B + B 64 x 256 B = 32 KiB each, 128 KiB of LDS); stage t+3 is requested while
+//               64 k-bytes (A 256 x 64 B + B 64 x 256 B = 32 KiB each, 128 KiB of LDS); stage t+4 is requested while
 //               stage t feeds the matrix cores, tracked with vmcnt (4 requests per lane and stage)
 //   LDS layout  16-byte chunks, placed so that every fragment read is bank-conflict free:
 //                 A (k contiguous): chunk (row r, c) at r*4 + (c ^ ((r>>2)&3))       -> ds_read_b128
@@ -20,7 +20,7 @@
 //               the permutation is applied on the global-address side (each lane fetches the chunk that belongs at its
 //               LDS position), the DMA itself writes lanes in order
 //   schedule    one barrier per stage, placed right after an MFMA issue; every fragment register is refilled from
-//               stage t+1 right after its last use in stage t, the 4 DMA requests of stage t+3 ride along
+//               stage t+1 right after its last use in stage t, the 4 DMA requests of stage t+4 ride along
 //   epilogue    the MFMA takes the B fragment as its first operand, so a lane's accumulator registers run along the
 //               output row: one v_permlane32_swap per register pair gives every lane 16 consecutive columns, written
 //               with 16-byte stores (bf16 through v_cvt_pk_bf16_f32 with an exact fall-back for NaN / inf / overflow)

@@ -232,8 +232,14 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                     g_t[2]++;
                 }
             }
+            gather_offsets();
         }
-        gather_offsets();
+        else
+        {
+            // same tap, next channels: the common case costs two scalar additions
+            g_delta_a += FBK;
+            g_delta_b += FBK;
+        }
     };
     if constexpr (GATHER)
     {
@@ -347,7 +353,9 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             read_b_tr16(f, j, st, wn, lane);
     };
 
-    for (int t = 0; t < FNST - 1; t++)
+    // all four slots of the ring are requested up front: a slot is free again as soon as its stage has been copied into
+    // fragment registers, which happens one step before the stage is multiplied
+    for (int t = 0; t < FNST; t++)
     {
 #pragma unroll
         for (int u = 0; u < 2; u++)
@@ -357,7 +365,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         }
     }
     // s_waitcnt immediate (gfx9): vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-    __builtin_amdgcn_s_waitcnt(0x0F78); // vmcnt(8): stage 0 has landed
+    __builtin_amdgcn_s_waitcnt(0x0F7C); // vmcnt(12): stage 0 has landed
     __syncthreads();
     auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
     {
@@ -403,19 +411,20 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #define RB(j) \
     if (RN) read_b(f, j, st);
 #define LA(u) \
-    if (LOADS) issue_a(u, t + FNST - 1, slot);
+    if (LOADS) issue_a(u, t + FNST, slot);
 #define LB(u) \
-    if (LOADS) issue_b(u, t + FNST - 1, slot);
+    if (LOADS) issue_b(u, t + FNST, slot);
     // One stage: 8 MFMAs; after the first one wait until stage t+1 has landed in every wavefront's view (WAITC leaves the
-    // younger stage in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
-    // other wavefront on the SIMD covers the tail of that latency); request stage t+3.
+    // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
+    // other wavefront on the SIMD covers the tail of that latency); request stage t+4 into the slot of stage t, whose
+    // fragments every wavefront read during the previous step (the barrier above orders those reads before this request).
     auto step = [&](int t, auto waitc, auto loads, auto readnext) __attribute__((always_inline))
     {
         constexpr int  WAITC = decltype(waitc)::value;
         constexpr bool LOADS = decltype(loads)::value;
         constexpr bool RN = decltype(readnext)::value;
         const char*    st = lds + ((t + 1) % FNST) * FSTAGE;
-        const int      slot = (t + FNST - 1) % FNST;
+        const int      slot = t % FNST;
         MMA(0, 0);
         FENCE;
         if (RN)
@@ -433,19 +442,20 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         RB(0) LB(1) MMA(3, 1); FENCE;
         RA(3) RB(1) FENCE;
     };
-    using W8 = std::integral_constant<int, 0x0F74>; // vmcnt(4): one stage of this wavefront's requests may still be in flight
+    using W8 = std::integral_constant<int, 0x0F78>; // vmcnt(8): two stages of this wavefront's requests may still be in flight
+    using W4 = std::integral_constant<int, 0x0F74>; // vmcnt(4): one stage
     using W0 = std::integral_constant<int, 0x0F70>; // vmcnt(0)
     using T = std::true_type;
     using F = std::false_type;
     int t = 0;
-    for (; t + 5 <= nk; t += 2)
+    for (; t + 5 <= nk; t += 2) // steps 0 .. nk-5 request stages 4 .. nk-1
     {
         step(t, W8 {}, T {}, T {});
         step(t + 1, W8 {}, T {}, T {});
     }
-    // t == nk - 4 (nk is even and >= 6)
-    step(t, W8 {}, T {}, T {});     // requests the last stage
-    step(t + 1, W8 {}, F {}, T {}); // stage nk-2 needed, stage nk-1 may be in flight
+    // t == nk - 4 (nk is even and >= 6): everything has been requested
+    step(t, W8 {}, F {}, T {});     // stage nk-3 needed, stages nk-2 and nk-1 may be in flight
+    step(t + 1, W4 {}, F {}, T {}); // stage nk-2 needed, stage nk-1 may be in flight
     step(t + 2, W0 {}, F {}, T {});
     step(t + 3, W0 {}, F {}, F {});
 #undef MMA
