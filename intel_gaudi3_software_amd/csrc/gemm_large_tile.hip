@@ -111,6 +111,7 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 } // namespace
 
 hipError_t launch_gemm_large_tile_f16(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_f16.hip
+hipError_t launch_gemm_large_tile_128(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_128.hip
 
 bool gemm_large_tile_applicable(const GemmProblem& p)
 {
@@ -118,6 +119,9 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     const bool two_byte = p.dtype == DT_BF16 || p.dtype == DT_FP16;
     const int  es = two_byte ? 2 : 1;
     const bool gather = p.A.kind == VIEW_CONV;
+    const int  tm = p.tile_m == 128 ? 128 : FBM;
+    // the 128-row tile: 2-byte operands, A staged k-contiguous (plain rows, or the fwd / dedx gather)
+    if (tm == 128 && (!two_byte || !p.A.k_contig || (gather && !p.A.pix_is_f))) return false;
     if (gather)
     {
         // bf16 / fp16, at most 32 taps, one problem per launch
@@ -144,7 +148,7 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     if (!p.A.vec_ok || !p.B.vec_ok) return false;
     if (!p.A.k_contig && !two_byte) return false; // f-contiguous A: bf16 / fp16 only
     if (gather && p.A.pix_is_f && !p.A.k_contig) return false;
-    if ((!gather && p.M % FBM) || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
+    if ((!gather && p.M % tm) || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
     if (p.split_k > 1)
     {
         // every slice an even number of stages, at least 6
@@ -164,12 +168,26 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     return true;
 }
 
+int gemm_fast_pick_tile_m(const GemmProblem& p, int num_cus)
+{
+    GemmProblem q = p;
+    q.split_k = 1;
+    q.tile_m = 128;
+    if (!gemm_large_tile_applicable(q)) return 0;
+    q.tile_m = 0;
+    if (!gemm_large_tile_applicable(q)) return 128; // M is a multiple of 128 only
+    // with at most half of the compute units busy, halving the tile doubles the workgroups without a second round
+    const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
+    return 2 * tiles <= num_cus ? 128 : 0;
+}
+
 int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
 {
     GemmProblem q = p;
     q.split_k = 1;
     if (!gemm_large_tile_applicable(q)) return 0;
-    const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
+    const int       tm = p.tile_m == 128 ? 128 : FBM;
+    const long long tiles = (long long) ((p.M + tm - 1) / tm) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
     const int       nk = p.K * dt_bytes(p.dtype) / FBK;
     int             best = 1;
     // Splitting the reduction pays when the tiles leave most of the chip idle and the reduction is long: a slice costs a
@@ -196,7 +214,9 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
 hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
-    dim3            grid(((p.M + FBM - 1) / FBM) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    const int       tm = p.tile_m == 128 ? 128 : FBM;
+    dim3            grid(((p.M + tm - 1) / tm) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    if (tm == 128) return launch_gemm_large_tile_128(p, grid, s);
     if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return launch_conv_bf16(p, grid, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);

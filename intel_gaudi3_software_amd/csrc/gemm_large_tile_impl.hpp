@@ -32,9 +32,10 @@ struct Frags
     v8i a[4], b[2];
 };
 
-__device__ __forceinline__ void read_a(Frags& f, int i, const char* st, int wm, int lane)
+// (row0: first row of this wavefront's block of the staged A tile; the B readers take the address of the stage's B part)
+__device__ __forceinline__ void read_a(Frags& f, int i, const char* st, int row0, int lane)
 {
-    const int r = wm * 128 + i * 32 + (lane & 31), c0 = 2 * (lane >> 5);
+    const int r = row0 + i * 32 + (lane & 31), c0 = 2 * (lane >> 5);
     const v4i lo = *(const v4i*) (st + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + fa_pos(r, c0 + 1) * 16);
     f.a[i] = v8i {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
@@ -48,7 +49,7 @@ __device__ __forceinline__ void read_b_tr(Frags& f, int j, const char* st, int w
     for (int tt = 0; tt < 4; tt++)
     {
         const int k = g * 32 + 8 * tt + rr;
-        t[tt] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS3 v2i*) (st + FBM * FBK + fb_pos(k, cb) * 16 + h * 8));
+        t[tt] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS3 v2i*) (st + fb_pos(k, cb) * 16 + h * 8));
     }
     f.b[j] = v8i {t[0].x, t[0].y, t[1].x, t[1].y, t[2].x, t[2].y, t[3].x, t[3].y};
 }
@@ -71,7 +72,7 @@ __device__ __forceinline__ void read_b_tr16(Frags& f, int j, const char* st, int
     {
         // reads 0, 1 -> k = 16 h + 0 .. 7 (first MFMA), reads 2, 3 -> k = 16 h + 8 .. 15 (second MFMA)
         const int k = 16 * h + 4 * tt + (q >> 2);
-        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + FBM * FBK + k * 512 + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
+        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + k * 512 + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
     }
     f.b[j] = u.v;
 }
@@ -99,7 +100,7 @@ __device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int
 __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int wn, int lane)
 {
     const int r = wn * 64 + j * 32 + (lane & 31), c0 = 2 * (lane >> 5);
-    const v4i lo = *(const v4i*) (st + FBM * FBK + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + FBM * FBK + fa_pos(r, c0 + 1) * 16);
+    const v4i lo = *(const v4i*) (st + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + fa_pos(r, c0 + 1) * 16);
     f.b[j] = v8i {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
 
@@ -118,9 +119,18 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // 2 plain, f contiguous (the "atb" forms; bf16 only: the stage then holds 32 k-rows x 256 f like an n-contiguous B and is
 // read with ds_read_b64_tr_b16); 3 convolution view with pixels along k (dedw: f = tap * channels + channel is fixed per
 // lane, the pixel advances by 32 per stage and is decoded incrementally).
-template<int ES, int FMT, bool B_KC, int AMODE = 0>
+// TM: rows of the output tile, 256 or 128 (128 for problems whose 256-row tiles would leave most of the chip idle; only
+// with A staged k-contiguous, AMODE 0 and 1).  A wavefront then owns TM / 2 rows x 64 columns.
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
+    static_assert(TM == 256 || (TM == 128 && AMODE < 2), "the 128-row tile exists for k-contiguous A only");
+    constexpr int  WR = TM / 2;                   // rows per wavefront
+    constexpr int  NI = WR / 32;                  // A fragments (32-row blocks) per wavefront
+    constexpr int  NUA = TM / 128;                // A requests per lane and stage (16 rows x 64 bytes per wavefront and request)
+    constexpr int  A_BYTES = TM * FBK;            // A part of a stage; the B part follows
+    constexpr int  STAGE = A_BYTES + FBK * FBN;   // 32 KiB or 24 KiB
+    constexpr int  NREQ = NUA + 2;                // requests per lane and stage
     constexpr bool GATHER = AMODE == 1;           // tap masks + uniform tap offsets
     constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3; // the last row tile may be partial
     constexpr bool A_KC = AMODE < 2;
@@ -128,7 +138,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
-    const int tiles_n = g.N / FBN, tiles_m = (g.M + FBM - 1) / FBM;
+    const int tiles_n = g.N / FBN, tiles_m = (g.M + TM - 1) / TM;
     int       tm, tn;
     {
         const int b = blockIdx.x, T = tiles_m * tiles_n;
@@ -150,16 +160,16 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     const int       b1 = bz % g.batch[1], b2 = bz / g.batch[1];
     const long long a_off = b0 * g.A.batch_stride[0] + b1 * g.A.batch_stride[1] + b2 * g.A.batch_stride[2];
     const long long b_off = b0 * g.B.batch_stride[0] + b1 * g.B.batch_stride[1] + b2 * g.B.batch_stride[2];
-    const int       m0 = tm * FBM, n0 = tn * FBN;
+    const int       m0 = tm * TM, n0 = tn * FBN;
     const long long lda = (A_KC ? g.A.stride_f : g.A.stride_k) * ES; // bytes between rows of the staged A tile
     const long long ldb = (B_KC ? g.B.stride_f : g.B.stride_k) * ES;
     const uint8_t*  A = (const uint8_t*) g.A.base + a_off * ES;
     const uint8_t*  B = (const uint8_t*) g.B.base + b_off * ES;
     const uint32_t  lds_base = (uint32_t) (uintptr_t) lds;
 
-    v16f acc[4][2];
+    v16f acc[NI][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < NI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -174,10 +184,14 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     for (int u = 0; u < 2; u++)
     {
         const int t = wave * 2 + u;
+        ga[u] = nullptr;
         if constexpr (AMODE == 0)
         {
-            const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-            ga[u] = A + (size_t) (m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
+            if (u < NUA)
+            {
+                const int r = (wave * NUA + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
+                ga[u] = A + (size_t) (m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
+            }
         }
         if constexpr (AMODE == 2)
         {
@@ -245,9 +259,9 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     {
         const int ntaps = g.A.ktap[0] * g.A.ktap[1] * g.A.ktap[2];
 #pragma unroll
-        for (int u = 0; u < 2; u++)
+        for (int u = 0; u < NUA; u++)
         {
-            const int r = (wave * 2 + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
+            const int r = (wave * NUA + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
             const int pix = min(m0 + r, g.M - 1);
             const PixelPos pp = decode_pixel(g.A, pix);
             long long      off0 = 0;
@@ -257,8 +271,14 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             ga[u] = A + off0 * ES + c * 16;
             if (m0 + r < g.M)
                 for (int t = 0; t < ntaps; t++) tap_ok[u] |= (conv_offset(g.A, pp, t) >= 0 ? 1u : 0u) << t;
-            if (g.B.kind == VIEW_TAPPED) gb[u] = B + (size_t) (n0 + r) * ldb + c * 16;
         }
+        if (g.B.kind == VIEW_TAPPED)
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+            {
+                const int r = (wave * 2 + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
+                gb[u] = B + (size_t) (n0 + r) * ldb + c * 16;
+            }
         // first stage of this workgroup's k range
         const int k0 = kt_begin * stage_ch;
         g_tap = k0 / g.A.nch;
@@ -306,7 +326,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 off += (long long) pos * g.A.src_stride[d] * 2;
             }
             const uint8_t* src = ok ? A + off : (const uint8_t*) gf_zero_page;
-            dma16(src, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+            dma16(src, lds_base + slot * STAGE + (wave * 2 + u) * 1024);
             // next stage: 32 pixels further
             int carry = 32;
 #pragma unroll
@@ -323,34 +343,34 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             w_pc[u][3] += carry;
         }
         else if constexpr (AMODE == 2)
-            dma16(ga[u] + (size_t) stage * (FBK / ES) * lda, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+            dma16(ga[u] + (size_t) stage * (FBK / ES) * lda, lds_base + slot * STAGE + (wave * 2 + u) * 1024);
         else if constexpr (GATHER)
         {
             const bool     ok = (tap_ok[u] >> g_tap) & 1u;
             const uint8_t* src = ok ? ga[u] + g_delta_a : (const uint8_t*) gf_zero_page;
-            dma16(src, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+            dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
         }
         else
-            dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * FSTAGE + (wave * 2 + u) * 1024);
+            dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
     };
     auto issue_b = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
         if (GATHER && g.B.kind == VIEW_TAPPED)
         {
-            dma16(gb[u] + g_delta_b, lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
+            dma16(gb[u] + g_delta_b, lds_base + slot * STAGE + A_BYTES + (wave * 2 + u) * 1024);
             if (u == 1) gather_advance(); // the stage's last request
             return;
         }
-        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * FSTAGE + FBM * FBK + (wave * 2 + u) * 1024);
+        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * STAGE + A_BYTES + (wave * 2 + u) * 1024);
         if (GATHER && u == 1) gather_advance();
     };
     auto read_b = [&](Frags & f, int j, const char* st) __attribute__((always_inline))
     {
-        if (B_KC) read_b_kc(f, j, st, wn, lane);
+        if (B_KC) read_b_kc(f, j, st + A_BYTES, wn, lane);
         else if (ES == 1)
-            read_b_tr(f, j, st, wn, lane);
+            read_b_tr(f, j, st + A_BYTES, wn, lane);
         else
-            read_b_tr16(f, j, st, wn, lane);
+            read_b_tr16(f, j, st + A_BYTES, wn, lane);
     };
 
     // all four slots of the ring are requested up front: a slot is free again as soon as its stage has been copied into
@@ -360,22 +380,22 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #pragma unroll
         for (int u = 0; u < 2; u++)
         {
-            issue_a(u, t, t);
+            if (u < NUA) issue_a(u, t, t);
             issue_b(u, t, t);
         }
     }
     // s_waitcnt immediate (gfx9): vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-    __builtin_amdgcn_s_waitcnt(0x0F7C); // vmcnt(12): stage 0 has landed
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * NREQ)); // three stages may still be in flight: stage 0 has landed
     __syncthreads();
     auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
     {
-        if constexpr (A_KC) read_a(fr, i, st, wm, lane);
+        if constexpr (A_KC) read_a(fr, i, st, wm * WR, lane);
         else
             read_a_tr16(fr, i, st, wm, lane);
     };
     Frags f;
 #pragma unroll
-    for (int i = 0; i < 4; i++) read_a_any(f, i, lds);
+    for (int i = 0; i < NI; i++) read_a_any(f, i, lds);
 #pragma unroll
     for (int j = 0; j < 2; j++) read_b(f, j, lds);
 
@@ -423,7 +443,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         constexpr int  WAITC = decltype(waitc)::value;
         constexpr bool LOADS = decltype(loads)::value;
         constexpr bool RN = decltype(readnext)::value;
-        const char*    st = lds + ((t + 1) % FNST) * FSTAGE;
+        const char*    st = lds + ((t + 1) % FNST) * STAGE;
         const int      slot = t % FNST;
         MMA(0, 0);
         FENCE;
@@ -434,17 +454,27 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         }
         FENCE;
         MMA(0, 1); FENCE;
-        RA(0) LA(0) MMA(1, 0); FENCE;
-        MMA(1, 1); FENCE;
-        RA(1) LA(1) MMA(2, 0); FENCE;
-        MMA(2, 1); FENCE;
-        RA(2) LB(0) MMA(3, 0); FENCE;
-        RB(0) LB(1) MMA(3, 1); FENCE;
-        RA(3) RB(1) FENCE;
+        if constexpr (NI == 4)
+        {
+            RA(0) LA(0) MMA(1, 0); FENCE;
+            MMA(1, 1); FENCE;
+            RA(1) LA(1) MMA(2, 0); FENCE;
+            MMA(2, 1); FENCE;
+            RA(2) LB(0) MMA(3, 0); FENCE;
+            RB(0) LB(1) MMA(3, 1); FENCE;
+            RA(3) RB(1) FENCE;
+        }
+        else
+        {
+            // 128-row tile: four MFMAs per stage, three requests
+            RA(0) LA(0) MMA(1, 0); FENCE;
+            RB(0) LB(0) MMA(1, 1); FENCE;
+            RA(1) RB(1) LB(1) FENCE;
+        }
     };
-    using W8 = std::integral_constant<int, 0x0F78>; // vmcnt(8): two stages of this wavefront's requests may still be in flight
-    using W4 = std::integral_constant<int, 0x0F74>; // vmcnt(4): one stage
-    using W0 = std::integral_constant<int, 0x0F70>; // vmcnt(0)
+    using W8 = std::integral_constant<int, 0x0F70 | (2 * NREQ)>; // two stages of this wavefront's requests may still be in flight
+    using W4 = std::integral_constant<int, 0x0F70 | NREQ>;       // one stage
+    using W0 = std::integral_constant<int, 0x0F70>;              // vmcnt(0)
     using T = std::true_type;
     using F = std::false_type;
     int t = 0;
@@ -480,8 +510,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
                            g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
     const int       kg = lane >> 5;
-    // element offset of this lane's first value in block (0, 0): row m0 + wm * 128 + lane % 32, column n0 + wn * 64 + 16 kg
-    const long long lane_elem = c_off + (long long) (m0 + wm * 128 + (lane & 31)) * ldc + n0 + wn * 64 + kg * 16;
+    // element offset of this lane's first value in block (0, 0): row m0 + wm * WR + lane % 32, column n0 + wn * 64 + 16 kg
+    const long long lane_elem = c_off + (long long) (m0 + wm * WR + (lane & 31)) * ldc + n0 + wn * 64 + kg * 16;
     // block (i, j) -> the lane's 16 values after the power-of-two factors and relu
     auto gather = [&](int i, int j, float (&val)[16]) __attribute__((always_inline))
     {
@@ -514,13 +544,13 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     auto walk = [&](auto store) __attribute__((always_inline))
     {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < NI; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
             {
                 float val[16];
                 gather(i, j, val);
-                if (!RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
+                if (!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
             }
     };
     typedef float    e_v4f __attribute__((ext_vector_type(4)));
@@ -531,14 +561,14 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     {
         // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
         float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N +
-                    (long long) (m0 + wm * 128 + (lane & 31)) * g.N + n0 + wn * 64 + kg * 16;
+                    (long long) (m0 + wm * WR + (lane & 31)) * g.N + n0 + wn * 64 + kg * 16;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < NI; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
             {
                 e_v4f*     o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
-                const bool row_ok = !RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M;
+                const bool row_ok = !RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M;
 #pragma unroll
                 for (int q = 0; q < 2; q++)
                 {
@@ -634,7 +664,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     {
         // rare cast settings: element-wise through the out-of-line generic converter (which applies relu itself)
 #pragma unroll 1
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < NI; i++)
 #pragma unroll 1
             for (int j = 0; j < 2; j++)
             {
@@ -647,7 +677,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                         // (dynamic block index: read the accumulators through a switch-free copy)
                         float lo = 0.0f, hi = 0.0f;
 #pragma unroll
-                        for (int ii = 0; ii < 4; ii++)
+                        for (int ii = 0; ii < NI; ii++)
 #pragma unroll
                             for (int jj = 0; jj < 2; jj++)
                                 if (ii == i && jj == j)
@@ -664,7 +694,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                     float x = val[c];
                     if (has_alpha) x *= alpha;
                     if (col_exp) x *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
-                    if (!RAGGED_M || m0 + wm * 128 + i * 32 + (lane & 31) < g.M) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
+                    if (!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
                 }
             }
     }
@@ -674,15 +704,16 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 
 // sets the dynamic-LDS limit once per kernel, then launches
 template<class K>
-hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s)
+hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s, int tile_m = FBM)
 {
+    const int lds_bytes = FNST * (tile_m * FBK + FBK * FBN);
     if (!attr_done)
     {
-        hipError_t e = hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, FNST * FSTAGE);
+        hipError_t e = hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(512), FNST * FSTAGE, s, p);
+    hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, s, p);
     return hipGetLastError();
 }
 } // namespace

@@ -320,6 +320,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         if (int rc = prepare_half_operands(h, g, ta, tb, a_base, b_base)) return rc;
     g.skip_flag = nullptr;
     g.skip_if = 0;
+    g.tile_m = gemm_fast_pick_tile_m(g, h->num_cus);
     g.split_k = gemm_pick_split_k(g, h->num_cus);
     g.workspace = nullptr;
     if (g.split_k > 1)

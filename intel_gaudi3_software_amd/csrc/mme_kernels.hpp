@@ -90,6 +90,7 @@ struct GemmProblem
     int          batch[3];
     OperandView  A, B;
     GemmEpilogue epi;
+    int          tile_m;     // large-tile kernel: rows of the output tile, 128 or 0 / 256 (chosen by gemm_fast_pick_tile_m)
     int          split_k;    // >1: partial sums go to workspace and are reduced in a fixed order
     float*       workspace;  // split_k * batch * M * N floats
     // device-side predicate: when skip_flag != NULL the whole launch returns at once if (*skip_flag == skip_epoch) == skip_if
@@ -102,6 +103,8 @@ struct GemmProblem
 
 size_t     gemm_workspace_bytes(const GemmProblem& p);
 int        gemm_pick_split_k(const GemmProblem& p, int num_cus);
+// 128 when the large-tile kernel should run this problem with 128-row tiles (few tiles, 2-byte operands, A k-contiguous), else 0
+int        gemm_fast_pick_tile_m(const GemmProblem& p, int num_cus);
 hipError_t launch_gemm(const GemmProblem& p, hipStream_t s);
 // large aligned fp8 problems (gemm_large_tile.hip); launch_gemm routes to it when applicable
 bool       gemm_large_tile_applicable(const GemmProblem& p);

@@ -129,3 +129,60 @@ def test_c5_batched_mixed_fp8_gemm_full_size(calc, orc):
         gf, wf = decode_fp8(orc, g, abi.FP8_143, 7), decode_fp8(orc, want, abi.FP8_143, 7)
         assert rel_frobenius(gf, wf) <= 3e-2
         assert np.count_nonzero(want & 0x7F) > rows * N // 2  # the slab is not a field of zeros
+
+
+@pytest.mark.parametrize("dt", [abi.BF16, abi.FP16])
+def test_large_tile_kernel_both_tile_heights(calc, orc, dt):
+    """The large-tile kernel picks 128-row tiles when 256-row tiles would occupy at most half of the compute units, else
+    256-row ones.  A bf16 / fp16 GEMM with 144 tiles of 256 x 256 (the 256-row kernel) and one with M = 384 (the 128-row
+    kernel; M is not a multiple of 256): slabs of rows against the oracle."""
+    import torch
+    rng = np.random.default_rng(3)
+    for (M, N, K) in [(3072, 3072, 320), (384, 512, 448)]:
+        if dt == abi.BF16:
+            a, b = (to_bf16_bits(rng.standard_normal(n).astype(np.float32)) for n in (M * K, N * K))
+        else:
+            a, b = (rng.standard_normal(n).astype(np.float16).view(np.uint16) for n in (M * K, N * K))
+        bias = 15 if dt == abi.FP16 else 0
+        out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, dt, _dev(a), bias), MmeSimTensor([K, N], 2, dt, _dev(b), bias),
+                         abi.OP_ABT)
+        calc.synchronize()
+        got = out.cpu().numpy().reshape(M, N)
+        for r0 in (0, M // 2 - 32, M - 64):
+            slab = np.ascontiguousarray(a.reshape(M, K)[r0:r0 + 64])
+            want = np.zeros(64 * N, np.float32)
+            da, db, do = desc(slab, [K, 64], dt, bias), desc(b, [K, N], dt, bias), desc(want, [N, 64], abi.FP32)
+            assert orc.orc_batch_gemm(A(do), A(da), A(db), abi.OP_ABT) == 0
+            assert rel_frobenius(got[r0:r0 + 64].ravel(), want) <= 1e-4, (M, r0)
+
+
+def test_conv_gather_with_256_row_tiles(calc, orc):
+    """A 3 x 3 forward convolution and dedx with enough pixels for more than 128 tiles of 256 rows (43 images of 28 x 28, 256
+    channels: 132 tiles), so that the gather runs on the 256-row kernel; first and last image against the oracle."""
+    import torch
+    rng = np.random.default_rng(4)
+    B, H, W, Cc, Kk = 43, 28, 28, 256, 256
+    xs, ws, ys = [Cc, W, H, 1, B], [Kk, Cc, 3, 3, 1], [Kk, W, H, 1, B]
+    x = to_bf16_bits(rng.standard_normal(int(np.prod(xs))).astype(np.float32))
+    w = to_bf16_bits((rng.standard_normal(int(np.prod(ws))) * 0.02).astype(np.float32))
+    dy = to_bf16_bits(rng.standard_normal(int(np.prod(ys))).astype(np.float32))
+    cp = ConvolutionParams(2, [1, 1, 0, 0])
+    p = abi.make_conv_params(2, (1, 1, 0), (1, 1, 1), (1, 1, 1))
+    X, Wt, DY = MmeSimTensor(xs, 5, abi.BF16, _dev(x)), MmeSimTensor(ws, 5, abi.BF16, _dev(w)), MmeSimTensor(ys, 5, abi.BF16, _dev(dy))
+    gy = torch.zeros(int(np.prod(ys)), dtype=torch.float32, device="cuda")
+    gdx = torch.zeros(int(np.prod(xs)), dtype=torch.float32, device="cuda")
+    out_y = MmeSimTensor(ys, 5, abi.FP32, gy)
+    calc.doConvolution(out_y, X, Wt, out_y, cp, abi.OP_FWD)
+    calc.doConvolution(MmeSimTensor(xs, 5, abi.FP32, gdx), X, Wt, DY, cp, abi.OP_DEDX)
+    calc.synchronize()
+    per_x, per_y = H * W * Cc, H * W * Kk
+    yg, dxg = gy.cpu().numpy().reshape(B, per_y), gdx.cpu().numpy().reshape(B, per_x)
+    for b in (0, B - 1):
+        xb, yb = np.ascontiguousarray(x[b * per_x:(b + 1) * per_x]), np.ascontiguousarray(dy[b * per_y:(b + 1) * per_y])
+        want_y, want_dx = np.zeros(per_y, np.float32), np.zeros(per_x, np.float32)
+        dxb, dwd = desc(xb, [Cc, W, H, 1, 1], abi.BF16), desc(w, ws, abi.BF16)
+        doy, dox, dyb = desc(want_y, [Kk, W, H, 1, 1], abi.FP32), desc(want_dx, [Cc, W, H, 1, 1], abi.FP32), desc(yb, [Kk, W, H, 1, 1], abi.BF16)
+        assert orc.orc_convolution(A(doy), A(dxb), A(dwd), A(doy), A(p), abi.OP_FWD, 0) == 0
+        assert orc.orc_convolution(A(dox), A(dox), A(dwd), A(dyb), A(p), abi.OP_DEDX, 0) == 0
+        assert rel_frobenius(yg[b], want_y) <= 1e-4 and rel_frobenius(dxg[b], want_dx) <= 1e-4
