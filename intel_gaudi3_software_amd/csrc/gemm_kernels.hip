@@ -15,29 +15,71 @@ void launch_gemm_fp8_11(const GemmProblem& p, dim3 grid, hipStream_t s);
 
 namespace
 {
-// sums the split-k partials in slice order (deterministic) and applies the epilogue
+// sums the split-k partials in slice order (deterministic) and applies the epilogue.  Four consecutive columns per lane
+// (16-byte loads, one per slice, issued four slices at a time) when N is a multiple of 4; the sum of an element is formed
+// in the same order either way.
 __global__ __launch_bounds__(THREADS) void splitk_reduce_kernel(GemmProblem g_by_value)
 {
     (void) g_by_value;
     KARG GemmProblem& g = *(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr();
     if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
+    typedef float r_v4f __attribute__((ext_vector_type(4)));
     const long long mn = (long long) g.M * g.N;
     const long long nb = (long long) g.batch[0] * g.batch[1] * g.batch[2];
     const long long total = mn * nb;
-    for (long long i = (long long) blockIdx.x * THREADS + threadIdx.x; i < total; i += (long long) gridDim.x * THREADS)
+    const int       S = g.split_k;
+    auto finish = [&](long long b, long long r, int count, const float* x) __attribute__((always_inline))
     {
-        const long long b = i / mn, r = i - b * mn;
-        float           x = 0.0f;
-        for (int z = 0; z < g.split_k; z++) x += g.workspace[(z * nb + b) * mn + r];
         const int m = (int) (r / g.N), n = (int) (r - (long long) m * g.N);
         int       bz = (int) b;
         const int b0 = bz % g.batch[0];
         bz /= g.batch[0];
         const int       b1 = bz % g.batch[1], b2 = bz / g.batch[1];
         const long long c_off = b0 * g.epi.batch_stride[0] + b1 * g.epi.batch_stride[1] + b2 * g.epi.batch_stride[2];
-        if (g.epi.has_alpha) x *= g.epi.alpha;
-        if (g.epi.col_exp) x *= pow2_of(g.epi.col_exp[n]);
-        store_out(g.epi, c_off + (long long) m * g.epi.ld + n, x);
+        const long long idx = c_off + (long long) m * g.epi.ld + n;
+        float           v[4];
+        for (int c = 0; c < count; c++)
+        {
+            v[c] = x[c];
+            if (g.epi.has_alpha) v[c] *= g.epi.alpha;
+            if (g.epi.col_exp) v[c] *= pow2_of(g.epi.col_exp[n + c]);
+        }
+        if (count == 4 && !g.epi.fused && (idx & 3) == 0 && ((uintptr_t) g.epi.out & 15u) == 0)
+            *(r_v4f*) ((float*) g.epi.out + idx) = r_v4f {v[0], v[1], v[2], v[3]};
+        else
+            for (int c = 0; c < count; c++) store_out(g.epi, idx + c, v[c]);
+    };
+    if ((g.N & 3) == 0 && ((uintptr_t) g.workspace & 15u) == 0)
+    {
+        const long long groups = total >> 2; // a group of four columns never crosses a row
+        for (long long q = (long long) blockIdx.x * THREADS + threadIdx.x; q < groups; q += (long long) gridDim.x * THREADS)
+        {
+            const long long i = q << 2, b = i / mn, r = i - b * mn;
+            const r_v4f*    w = (const r_v4f*) (g.workspace + b * mn + r);
+            const long long step = nb * mn / 4; // r_v4f elements between slices
+            r_v4f           x = {0.0f, 0.0f, 0.0f, 0.0f};
+            int             z = 0;
+            for (; z + 4 <= S; z += 4)
+            {
+                const r_v4f p0 = __builtin_nontemporal_load(w + (z + 0) * step), p1 = __builtin_nontemporal_load(w + (z + 1) * step),
+                            p2 = __builtin_nontemporal_load(w + (z + 2) * step), p3 = __builtin_nontemporal_load(w + (z + 3) * step);
+                x += p0;
+                x += p1;
+                x += p2;
+                x += p3;
+            }
+            for (; z < S; z++) x += __builtin_nontemporal_load(w + z * step);
+            const float xs[4] = {x.x, x.y, x.z, x.w};
+            finish(b, r, 4, xs);
+        }
+        return;
+    }
+    for (long long i = (long long) blockIdx.x * THREADS + threadIdx.x; i < total; i += (long long) gridDim.x * THREADS)
+    {
+        const long long b = i / mn, r = i - b * mn;
+        float           x = 0.0f;
+        for (int z = 0; z < S; z++) x += g.workspace[(z * nb + b) * mn + r];
+        finish(b, r, 1, &x);
     }
 }
 
