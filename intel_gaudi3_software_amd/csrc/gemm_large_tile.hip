@@ -120,8 +120,8 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     const int  es = two_byte ? 2 : 1;
     const bool gather = p.A.kind == VIEW_CONV;
     const int  tm = p.tile_m == 128 ? 128 : FBM;
-    // the 128-row tile: 2-byte operands, A staged k-contiguous (plain rows, or the fwd / dedx gather)
-    if (tm == 128 && (!two_byte || !p.A.k_contig || (gather && !p.A.pix_is_f))) return false;
+    // the 128-row tile: 2-byte operands; A plain rows, the fwd / dedx gather, or dedw's pixels-along-k view
+    if (tm == 128 && (!two_byte || (!p.A.k_contig && !(gather && !p.A.pix_is_f)))) return false;
     if (gather)
     {
         // bf16 / fp16, at most 32 taps, one problem per launch
@@ -194,7 +194,8 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
     // pass of the fp32 output through the workspace plus the reduction kernel.  Rough model in microseconds: a stage (128 bytes of
     // k per row) takes 1.0 as measured on full-size fp8 and bf16 problems, the workspace moves at 3 TB/s (the reduction
     // kernel's measured rate is 2.3 .. 3.1), the extra launch costs 6.  Every slice keeps an even number of stages, at least 6.
-    const double stage_us = 1.0;
+    // (0.75 per stage of a 128-row tile: half the matrix work, the same latencies)
+    const double stage_us = tm == 128 ? 0.75 : 1.0;
     const double out_bytes = 8.0 * p.M * (double) p.N * p.batch[0] * p.batch[1] * p.batch[2];
     const double t1 = (double) ((tiles + num_cus - 1) / num_cus) * nk * stage_us;
     double       best_t = 0.8 * t1; // a split has to promise a clear gain

@@ -77,11 +77,13 @@ __device__ __forceinline__ void read_b_tr16(Frags& f, int j, const char* st, int
     f.b[j] = u.v;
 }
 
-// bf16, A stored f-contiguous: the same stage layout and reads as an n-contiguous B, over the wavefront's 128 rows
+// bf16, A stored f-contiguous: the same stage layout and reads as an n-contiguous B, over the wavefront's TM / 2 rows
+// (a k-row of the stage is TM elements = TM / 16 blocks of 32 bytes)
+template<int TM>
 __device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int wm, int lane)
 {
     typedef short v4s __attribute__((ext_vector_type(4)));
-    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wm * 8 + i * 2 + (g & 1);
+    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wm * (TM / 32) + i * 2 + (g & 1);
     union
     {
         v4s h4[4];
@@ -91,7 +93,7 @@ __device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int
     for (int tt = 0; tt < 4; tt++)
     {
         const int k = 16 * h + 4 * tt + (q >> 2);
-        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + k * 512 + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
+        u.h4[tt] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS3 v4s*) (st + k * (TM * 2) + ((block ^ (k & 3)) << 5) + ((q & 3) << 3)));
     }
     f.a[i] = u.v;
 }
@@ -119,12 +121,13 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // 2 plain, f contiguous (the "atb" forms; bf16 only: the stage then holds 32 k-rows x 256 f like an n-contiguous B and is
 // read with ds_read_b64_tr_b16); 3 convolution view with pixels along k (dedw: f = tap * channels + channel is fixed per
 // lane, the pixel advances by 32 per stage and is decoded incrementally).
-// TM: rows of the output tile, 256 or 128 (128 for problems whose 256-row tiles would leave most of the chip idle; only
-// with A staged k-contiguous, AMODE 0 and 1).  A wavefront then owns TM / 2 rows x 64 columns.
+// TM: rows of the output tile, 256 or 128 (128 for problems whose 256-row tiles would leave most of the chip idle; AMODE
+// 0, 1 and 3).  A wavefront then owns TM / 2 rows x 64 columns; an f-contiguous A stage is 32 k-rows of TM elements, one
+// request of 16 bytes per lane covers 2 (TM 256) or 4 (TM 128) of them.
 template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
-    static_assert(TM == 256 || (TM == 128 && AMODE < 2), "the 128-row tile exists for k-contiguous A only");
+    static_assert(TM == 256 || (TM == 128 && AMODE != 2), "the 128-row tile is not instantiated for plain f-contiguous A");
     constexpr int  WR = TM / 2;                   // rows per wavefront
     constexpr int  NI = WR / 32;                  // A fragments (32-row blocks) per wavefront
     constexpr int  NUA = TM / 128;                // A requests per lane and stage (16 rows x 64 bytes per wavefront and request)
@@ -300,8 +303,10 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #pragma unroll
         for (int u = 0; u < 2; u++)
         {
-            const int kr = (wave * 2 + u) * 2 + (lane >> 5), chunk = (lane & 31) ^ ((kr & 3) << 1);
-            const int f = m0 + chunk * 8, tap = f / g.A.nch;
+            if (u >= NUA) break;
+            constexpr int RPQ = 512 / TM; // k-rows per request
+            const int     kr = (wave * NUA + u) * RPQ + lane / (64 / RPQ), chunk = (lane & (64 / RPQ - 1)) ^ ((kr & 3) << 1);
+            const int     f = m0 + chunk * 8, tap = f / g.A.nch;
             w_ch[u] = f < g.M ? (long long) (f - tap * g.A.nch) * 2 : -1;
             w_t[u][0] = tap % g.A.ktap[0];
             w_t[u][1] = (tap / g.A.ktap[0]) % g.A.ktap[1];
@@ -326,7 +331,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 off += (long long) pos * g.A.src_stride[d] * 2;
             }
             const uint8_t* src = ok ? A + off : (const uint8_t*) gf_zero_page;
-            dma16(src, lds_base + slot * STAGE + (wave * 2 + u) * 1024);
+            dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
             // next stage: 32 pixels further
             int carry = 32;
 #pragma unroll
@@ -391,7 +396,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     {
         if constexpr (A_KC) read_a(fr, i, st, wm * WR, lane);
         else
-            read_a_tr16(fr, i, st, wm, lane);
+            read_a_tr16<TM>(fr, i, st, wm, lane);
     };
     Frags f;
 #pragma unroll

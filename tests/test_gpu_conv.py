@@ -182,11 +182,14 @@ def test_conv_large_tile_gather_vs_oracle(calc, orc, case, op, dt, bias):
     assert rel_frobenius(got, want) <= 1e-4
 
 
-# dedw on the large-tile kernel: pixels (the reduction) a multiple of 64 and at least 192, K = 256 output columns
+# dedw on the large-tile kernel: pixels (the reduction) a multiple of 64 and at least 192, K a multiple of 256 output columns.
+# Up to 128 tiles of 256 x 256 the kernel runs with 128-row tiles (the first three cases), beyond that with 256-row ones
+# (the last case: 9 x 15 tiles).
 DEDW_CASES = [
     (256, 256, 8, 8, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),
     (64, 256, 16, 8, 1, 2, 3, 3, 1, (2, 2, 0), (1, 1, 1), (2, 2, 1), 2),     # M = 576: ragged row tile, three taps per tile
     (32, 256, 18, 17, 1, 1, 3, 3, 1, (0, 0, 0), (2, 2, 1), (1, 1, 1), 2),    # strided: 8 x 8 output pixels
+    (256, 3840, 8, 8, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),
 ]
 
 
