@@ -281,45 +281,9 @@ int fold_alpha(mme_hip_handle h, GemmEpilogue& e, int fold)
     return MME_HIP_OK;
 }
 
-// fp16 / ufp16 / tf32 operands.  Two fp16 operands in full inf/NaN mode are IEEE half with the exponent bias as a power of
-// two: they go to the fp16 matrix instruction as they are.  Every other combination (unsigned fp16 with its 6-bit
-// exponent, exponent-all-ones codes that are finite, tf32) is first turned into fp32 words holding the operands' exact
-// values (tf32: the rounded ones), in the operands' own layout, and contracted by the fp32 instantiation.
-int prepare_half_operands(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, const mme_hip_tensor* tb, const void* a_base, const void* b_base)
+// picks tile height and k-slices of a problem and makes sure the split-k workspace can hold its partial sums
+int plan_launch(mme_hip_handle h, GemmProblem& g)
 {
-    if (ta->dtype == MME_HIP_FP16 && tb->dtype == MME_HIP_FP16 && ta->inf_nan_mode == 0 && tb->inf_nan_mode == 0)
-    {
-        g.dtype = DT_FP16;
-        return fold_alpha(h, g.epi, (15 - (int) ta->fp_bias) + (15 - (int) tb->fp_bias));
-    }
-    const size_t na = span_elements(ta), nb = span_elements(tb);
-    const size_t na_pad = (na + 3) & ~(size_t) 3;
-    HIP_TRY(h, h->decode_ws.reserve((na_pad + nb + 4) * 4));
-    float* da = (float*) h->decode_ws.p;
-    float* db = da + na_pad;
-    const mme_hip_tensor* t[2] = {ta, tb};
-    const void*           src[2] = {a_base, b_base};
-    float*                dst[2] = {da, db};
-    const size_t          cnt[2] = {na, nb};
-    for (int i = 0; i < 2; i++)
-    {
-        if (t[i]->dtype == MME_HIP_TF32) HIP_TRY(h, launch_round_to_tf32(dst[i], src[i], cnt[i], h->operand_clip_fp, h->operand_clip_inf_in, h->stream));
-        else
-            HIP_TRY(h, launch_cast_to_fp32(dst[i], src[i], t[i]->dtype, (int) t[i]->fp_bias, t[i]->inf_nan_mode, cnt[i], 1.0f, 0, nullptr, 0, h->stream));
-    }
-    g.dtype = DT_FP32;
-    g.A.base = (const char*) da;
-    g.B.base = (const char*) db;
-    return MME_HIP_OK;
-}
-
-int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, const mme_hip_tensor* tb, const void* a_base,
-                    const void* b_base)
-{
-    if (is_fp16(g.dtype) || g.dtype == MME_HIP_TF32)
-        if (int rc = prepare_half_operands(h, g, ta, tb, a_base, b_base)) return rc;
-    g.skip_flag = nullptr;
-    g.skip_if = 0;
     g.tile_m = gemm_fast_pick_tile_m(g, h->num_cus);
     g.split_k = gemm_pick_split_k(g, h->num_cus);
     g.workspace = nullptr;
@@ -328,6 +292,139 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         HIP_TRY(h, h->split_ws.reserve(gemm_workspace_bytes(g)));
         g.workspace = (float*) h->split_ws.p;
     }
+    return MME_HIP_OK;
+}
+
+// fp16 / ufp16 / tf32 operands.  Two fp16 operands in full inf/NaN mode are IEEE half with the exponent bias as a power of
+// two: they go to the fp16 matrix instruction as they are (returns with g.dtype = DT_FP16, nothing launched).  Every other
+// combination (unsigned fp16 with its 6-bit exponent, exponent-all-ones codes that are finite, tf32) is contracted here:
+//  - plain GEMMs of some size: each operand is written as two bf16 parts that add up to its exact value and the bf16 kernels
+//    contract the 4 K long rows (split_bf16_kernel); operands that hold inf or NaN raise a device flag, which skips that
+//    contraction and lets the fp32 one below run instead, so the call never waits for the device;
+//  - everything else: fp32 words holding the operands' exact values (tf32: the rounded ones), in the operands' own layout,
+//    contracted by the fp32 instantiation.
+int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, const mme_hip_tensor* tb, const void* a_base, const void* b_base,
+                         bool& done)
+{
+    done = false;
+    if (ta->dtype == MME_HIP_FP16 && tb->dtype == MME_HIP_FP16 && ta->inf_nan_mode == 0 && tb->inf_nan_mode == 0)
+    {
+        g.dtype = DT_FP16;
+        return fold_alpha(h, g.epi, (15 - (int) ta->fp_bias) + (15 - (int) tb->fp_bias));
+    }
+    done = true;
+    const long long nbatch = (long long) g.batch[0] * g.batch[1] * g.batch[2];
+    const bool      two_part = g.A.kind == VIEW_PLAIN && g.B.kind == VIEW_PLAIN && (long long) g.M * g.N * g.K * nbatch >= (1ll << 26) &&
+                          g.K <= (1 << 28);
+    const size_t na = span_elements(ta), nb = span_elements(tb);
+    const size_t na_pad = (na + 3) & ~(size_t) 3;
+    size_t       part_elems[2] = {0, 0};
+    long long    eff[2][3];
+    OperandView* view[2] = {&g.A, &g.B};
+    const int    free_extent[2] = {g.M, g.N};
+    if (two_part)
+        for (int i = 0; i < 2; i++)
+        {
+            part_elems[i] = (size_t) free_extent[i] * g.K * 4;
+            for (int d = 0; d < 3; d++)
+            {
+                eff[i][d] = view[i]->batch_stride[d] ? g.batch[d] : 1;
+                part_elems[i] *= (size_t) eff[i][d];
+            }
+            part_elems[i] = (part_elems[i] + 7) & ~(size_t) 7;
+        }
+    HIP_TRY(h, h->decode_ws.reserve((na_pad + nb + 4) * 4 + (part_elems[0] + part_elems[1]) * 2));
+    float*    da = (float*) h->decode_ws.p;
+    float*    db = da + na_pad;
+    uint16_t* parts = (uint16_t*) (db + ((nb + 3) & ~(size_t) 3));
+    const mme_hip_tensor* t[2] = {ta, tb};
+    const void*           src[2] = {a_base, b_base};
+    uint32_t*             flag = nullptr;
+    uint32_t              epoch = 0;
+    GemmProblem           g2 = g;
+    if (two_part)
+    {
+        if (int rc = ensure_flag(h)) return rc;
+        flag = (uint32_t*) h->flag.p;
+        epoch = ++h->specials_epoch;
+        OperandView* v2[2] = {&g2.A, &g2.B};
+        uint16_t*    dst = parts;
+        for (int i = 0; i < 2; i++)
+        {
+            SplitBf16Args a;
+            a.F = free_extent[i];
+            a.K = g.K;
+            a.sf = view[i]->stride_f;
+            a.sk = view[i]->stride_k;
+            a.k_contig = view[i]->k_contig;
+            a.is_b = i;
+            a.bias = (int) t[i]->fp_bias;
+            a.mode = t[i]->inf_nan_mode;
+            a.clip = h->operand_clip_fp;
+            a.clip_inf_in = h->operand_clip_inf_in;
+            a.flag = flag;
+            a.epoch = epoch;
+            long long bstride[3], run = (long long) a.F * a.K * 4;
+            for (int d = 0; d < 3; d++)
+            {
+                a.e[d] = (int) eff[i][d];
+                a.bs[d] = view[i]->batch_stride[d];
+                bstride[d] = view[i]->batch_stride[d] ? run : 0;
+                run *= eff[i][d];
+            }
+            HIP_TRY(h, launch_split_bf16(dst, src[i], t[i]->dtype, a, h->stream));
+            if (a.k_contig) set_plain_view(*v2[i], dst, 4ll * a.K, 1, true, 2, 4 * a.K, bstride);
+            else
+                set_plain_view(*v2[i], dst, 1, a.F, false, 2, a.F, bstride);
+            dst += part_elems[i];
+        }
+        g2.dtype = DT_BF16;
+        g2.K = 4 * g.K;
+    }
+    // the fp32 contraction: the only one, or the one that runs when an operand holds inf / NaN
+    for (int i = 0; i < 2; i++)
+    {
+        float* d = i ? db : da;
+        if (t[i]->dtype == MME_HIP_TF32)
+            HIP_TRY(h, launch_round_to_tf32(d, src[i], i ? nb : na, h->operand_clip_fp, h->operand_clip_inf_in, h->stream, flag, epoch));
+        else
+            HIP_TRY(h, launch_cast_to_fp32(d, src[i], t[i]->dtype, (int) t[i]->fp_bias, t[i]->inf_nan_mode, i ? nb : na, 1.0f, 0, nullptr, 0, h->stream,
+                                           flag, epoch));
+    }
+    g.dtype = DT_FP32;
+    g.A.base = (const char*) da;
+    g.B.base = (const char*) db;
+    g.skip_flag = flag;
+    g.skip_epoch = epoch;
+    g.skip_if = 0; // runs when the flag holds this call's epoch
+    if (two_part)
+    {
+        // both contractions may slice k; size the shared workspace for the larger request before either is launched
+        GemmProblem probe = g;
+        if (int rc = plan_launch(h, probe)) return rc;
+        g2.skip_flag = flag;
+        g2.skip_epoch = epoch;
+        g2.skip_if = 1;
+        if (int rc = plan_launch(h, g2)) return rc; // (the workspace only grows: it now fits either request)
+        HIP_TRY(h, launch_gemm(g2, h->stream));
+    }
+    if (int rc = plan_launch(h, g)) return rc;
+    HIP_TRY(h, launch_gemm(g, h->stream));
+    return MME_HIP_OK;
+}
+
+int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, const mme_hip_tensor* tb, const void* a_base,
+                    const void* b_base)
+{
+    g.skip_flag = nullptr;
+    g.skip_if = 0;
+    if (is_fp16(g.dtype) || g.dtype == MME_HIP_TF32)
+    {
+        bool done = false;
+        if (int rc = run_half_contraction(h, g, ta, tb, a_base, b_base, done)) return rc;
+        if (done) return MME_HIP_OK;
+    }
+    if (int rc = plan_launch(h, g)) return rc;
     if (!is_fp8(g.dtype))
     {
         HIP_TRY(h, launch_gemm(g, h->stream));

@@ -339,3 +339,73 @@ def test_fp16_large_tile_every_k_position(calc, orc):
         ha, hb = a.astype(np.float16).view(np.uint16).ravel(), bmat.astype(np.float16).view(np.uint16).ravel()
         got, ref = _gemm_both(calc, orc, abi.OP_ABT if b_kc else abi.OP_AB, M, N, K, PAIRS[0], ha, hb)
         assert np.array_equal(got.reshape(M, N), want) and np.array_equal(ref.reshape(M, N), want)
+
+
+# ---- the two-part bf16 path: plain GEMMs of at least 2^26 multiply-adds whose operands are not both IEEE half ------------
+TWO_PART_PAIRS = PAIRS[2:]
+
+
+@pytest.mark.parametrize("op", OPS)
+@pytest.mark.parametrize("pair", TWO_PART_PAIRS)
+def test_two_part_path_vs_oracle(calc, orc, op, pair):
+    """Operands written as hi + lo bf16 parts and contracted over 4 K by the bf16 kernels: a shape for the large-tile kernel
+    and a ragged, batched one (B broadcast) for the general kernel, all four layouts."""
+    rng = np.random.default_rng(300 + op)
+    for (M, N, K, batch) in [(256, 256, 1024, (1, 1, 1)), (200, 136, 1237, (2, 1, 1))]:
+        nb = int(np.prod(batch))
+        a = _operand(rng, orc, pair[0], pair[2], pair[4], M * K * nb)
+        b = _operand(rng, orc, pair[1], pair[3], pair[5], N * K)
+        got, want = _gemm_both(calc, orc, op, M, N, K, pair, a, b, batch)
+        assert rel_frobenius(got, want) <= 1e-4, (M, N, K)
+
+
+@pytest.mark.parametrize("pair", [PAIRS[5], PAIRS[6]])
+def test_two_part_path_every_k_position(calc, orc, pair):
+    """One-hot operands whose values need all 11 significant bits (so both parts are non-zero) walk a single product through
+    every k position of the concatenated reduction; the products are exact."""
+    M, N, K = 256, 256, 1024
+    a = np.zeros((M, K), np.float32)
+    b = np.zeros((K, N), np.float32)
+    perm_m = np.random.default_rng(6).permutation(M)
+    for k in range(K):
+        a[perm_m[k % M], k] = 1025.0 + (k % 1000)          # 11 significant bits
+        b[k, (k * 11 + 2 + 64 * (k // M)) % N] = 1027.0 if k % 2 else 1.0
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(want.astype(np.float64), a.astype(np.float64) @ b.astype(np.float64))  # exactly representable
+    for b_kc in (False, True):
+        bmat = b.T.copy() if b_kc else b
+        if pair[0] == abi.TF32:
+            ha, hb = a.view(np.uint32).ravel().copy(), bmat.view(np.uint32).ravel().copy()
+        else:
+            ha, hb = _quant(orc, pair[0], pair[2], pair[4], a.ravel()), _quant(orc, pair[1], pair[3], pair[5], bmat.ravel())
+        got, ref = _gemm_both(calc, orc, abi.OP_ABT if b_kc else abi.OP_AB, M, N, K, pair, ha, hb)
+        assert np.array_equal(got.reshape(M, N), want) and np.array_equal(ref.reshape(M, N), want)
+
+
+@pytest.mark.parametrize("pair", [PAIRS[3], PAIRS[6]])
+def test_two_part_path_steps_aside_for_inf_and_nan(calc, orc, pair):
+    """inf * 0 would appear among the partial products of split operands: a call whose operands hold inf or NaN is contracted
+    from fp32 copies instead (decided on the device), and the next call without them takes the two-part path again."""
+    dtA, dtB, bA, bB, mA, mB = pair
+    rng = np.random.default_rng(10)
+    M, N, K = 256, 256, 1024
+    a = _operand(rng, orc, dtA, bA, mA, M * K)
+    b = _operand(rng, orc, dtB, bB, mB, N * K)
+    clean, want_clean = _gemm_both(calc, orc, abi.OP_ABT, M, N, K, pair, a, b)
+    a2 = a.copy()
+    if dtA == abi.TF32:
+        a2.reshape(M, K)[3, 5], a2.reshape(M, K)[7, 9] = 0x7F800000, 0x7FC00001
+        b.reshape(N, K)[2, 5] = 0  # inf * 0
+    else:
+        a2.reshape(M, K)[3, 5], a2.reshape(M, K)[7, 9] = 0x7C00, 0x7E01
+        b.reshape(N, K)[2, 5] = 0
+    got, want = _gemm_both(calc, orc, abi.OP_ABT, M, N, K, pair, a2, b)
+    assert np.isnan(want).any() and np.isinf(want).any()
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    inf = np.isinf(want)
+    assert np.array_equal(got[inf], want[inf])
+    fin = np.isfinite(want)
+    assert rel_frobenius(got[fin], want[fin]) <= 1e-4
+    assert rel_frobenius(clean, want_clean) <= 1e-4
+    again, want_again = _gemm_both(calc, orc, abi.OP_ABT, M, N, K, pair, a, b)
+    assert np.isfinite(again).all() and rel_frobenius(again, want_again) <= 1e-4
