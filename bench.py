@@ -246,26 +246,6 @@ def extra_measurements(calc, stream):
     t = timed(lambda: calc.doBatchGemm(Y1, A1, B1, abi.OP_AB))
     res["gemm_bf16_512x512x512_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n1 ** 3 / t / 1e12, "frac_bf16_peak": 2.0 * n1 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
     # fp16 (IEEE half through the fp16 matrix instruction) and ufp16 (decoded to fp32 first) 4096^3 -> fp32; fp32 -> fp16 cast
-    n4 = 4096
-    h16 = lambda: torch.randn(n4 * n4, device="cuda").to(torch.float16).view(torch.int16)
-    AH, BH = MmeSimTensor([n4, n4], 2, abi.FP16, h16(), 15), MmeSimTensor([n4, n4], 2, abi.FP16, h16(), 15)
-    YH = MmeSimTensor([n4, n4], 2, abi.FP32, torch.zeros(n4 * n4, dtype=torch.float32, device="cuda"))
-    t = timed(lambda: calc.doBatchGemm(YH, AH, BH, abi.OP_ABT), n=20)
-    res["gemm_fp16_4096x4096x4096_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n4 ** 3 / t / 1e12, "frac_fp16_peak": 2.0 * n4 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
-    u16 = lambda: torch.randint(0x7000, 0x8800, (n4 * n4,), dtype=torch.int32, device="cuda").to(torch.int16)
-    AU, BU = MmeSimTensor([n4, n4], 2, abi.UFP16, u16(), 31), MmeSimTensor([n4, n4], 2, abi.UFP16, u16(), 31)
-    t = timed(lambda: calc.doBatchGemm(YH, AU, BU, abi.OP_ABT), n=10, warm=2)
-    # unsigned fp16 runs as a bf16 contraction over 4 K (operands split into two bf16 parts): TFLOP/s counts the algorithm's
-    # 2 M N K, the fraction prices the four bf16 products per multiply-add that the matrix cores execute
-    res["gemm_ufp16_4096x4096x4096_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n4 ** 3 / t / 1e12,
-                                                 "frac_bf16_peak_of_issued_products": 4 * 2.0 * n4 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
-    del AH, BH, AU, BU, YH
-    nc = 1 << 28
-    xc = torch.randn(nc, device="cuda")
-    oc = torch.zeros(nc, dtype=torch.int16, device="cuda")
-    t = timed(lambda: calc.castFromFp32(oc, abi.FP16, xc, nc, fpBias=15, clipFp=True), n=20)
-    res["cast_fp32_to_fp16"] = {"seconds": t, "GB/s": nc * 6 / t / 1e9, "frac_hbm_peak": nc * 6 / t / 1e9 / PEAK_HBM_GBS}
-    del xc, oc
     # c4: bf16 3x3 dedx / dedw, N=32 28x28 C=K=256
     Cc = Kk = 256
     H = Wd = 28
@@ -294,6 +274,27 @@ def extra_measurements(calc, stream):
     fl = 2.0 * b5 * M5 * N5 * K5
     t = timed(lambda: calc.doBatchGemm(Y5, A5, B5, abi.OP_AB, epilogue=e5), n=10, warm=2)
     res["bgemm_fp8_143x152_4x2048x14336x4096_fp8_out"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
+    # the fp16 flavours last: their work spaces (two bf16 copies of both operands) are the largest allocations of the run
+    n4 = 4096
+    h16 = lambda: torch.randn(n4 * n4, device="cuda").to(torch.float16).view(torch.int16)
+    AH, BH = MmeSimTensor([n4, n4], 2, abi.FP16, h16(), 15), MmeSimTensor([n4, n4], 2, abi.FP16, h16(), 15)
+    YH = MmeSimTensor([n4, n4], 2, abi.FP32, torch.zeros(n4 * n4, dtype=torch.float32, device="cuda"))
+    t = timed(lambda: calc.doBatchGemm(YH, AH, BH, abi.OP_ABT), n=20)
+    res["gemm_fp16_4096x4096x4096_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n4 ** 3 / t / 1e12, "frac_fp16_peak": 2.0 * n4 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
+    u16 = lambda: torch.randint(0x7000, 0x8800, (n4 * n4,), dtype=torch.int32, device="cuda").to(torch.int16)
+    AU, BU = MmeSimTensor([n4, n4], 2, abi.UFP16, u16(), 31), MmeSimTensor([n4, n4], 2, abi.UFP16, u16(), 31)
+    t = timed(lambda: calc.doBatchGemm(YH, AU, BU, abi.OP_ABT), n=10, warm=2)
+    # unsigned fp16 runs as a bf16 contraction over 4 K (operands split into two bf16 parts): TFLOP/s counts the algorithm's
+    # 2 M N K, the fraction prices the four bf16 products per multiply-add that the matrix cores execute
+    res["gemm_ufp16_4096x4096x4096_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n4 ** 3 / t / 1e12,
+                                                 "frac_bf16_peak_of_issued_products": 4 * 2.0 * n4 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
+    del AH, BH, AU, BU, YH
+    nc = 1 << 28
+    xc = torch.randn(nc, device="cuda")
+    oc = torch.zeros(nc, dtype=torch.int16, device="cuda")
+    t = timed(lambda: calc.castFromFp32(oc, abi.FP16, xc, nc, fpBias=15, clipFp=True), n=20)
+    res["cast_fp32_to_fp16"] = {"seconds": t, "GB/s": nc * 6 / t / 1e9, "frac_hbm_peak": nc * 6 / t / 1e9 / PEAK_HBM_GBS}
+    del xc, oc
     return res
 
 

@@ -112,6 +112,14 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 
 hipError_t launch_gemm_large_tile_f16(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_f16.hip
 hipError_t launch_gemm_large_tile_128(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_128.hip
+hipError_t launch_gemm_large_tile_ragged(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged.hip
+
+// the shape is not made of whole tiles (the pixel rows of a convolution view do not count: every kernel handles those)
+static bool large_tile_ragged(const GemmProblem& p)
+{
+    const int tm = p.tile_m == 128 ? 128 : FBM;
+    return (p.A.kind != VIEW_CONV && p.M % tm != 0) || p.N % FBN != 0;
+}
 
 bool gemm_large_tile_applicable(const GemmProblem& p)
 {
@@ -148,7 +156,13 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     if (!p.A.vec_ok || !p.B.vec_ok) return false;
     if (!p.A.k_contig && !two_byte) return false; // f-contiguous A: bf16 / fp16 only
     if (gather && p.A.pix_is_f && !p.A.k_contig) return false;
-    if ((!gather && p.M % tm) || p.N % FBN || (p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
+    // whole tiles, except: the convolution views take any pixel count, and the GEMM forms with A k-contiguous have kernels for
+    // partial tiles (any M from 64, N a multiple of 16 from 128: a lane's 16 output columns are then all in or all out)
+    if (large_tile_ragged(p))
+    {
+        if (gather || !p.A.k_contig || p.M < 64 || p.N % 16 || p.N < FBN / 2) return false;
+    }
+    if ((p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
     if (p.split_k > 1)
     {
         // every slice an even number of stages, at least 6
@@ -175,9 +189,9 @@ int gemm_fast_pick_tile_m(const GemmProblem& p, int num_cus)
     q.tile_m = 128;
     if (!gemm_large_tile_applicable(q)) return 0;
     q.tile_m = 0;
-    if (!gemm_large_tile_applicable(q)) return 128; // M is a multiple of 128 only
+    if (!gemm_large_tile_applicable(q)) return 128; // (A contiguous along its rows, M a multiple of 128 only)
     // with at most half of the compute units busy, halving the tile doubles the workgroups without a second round
-    const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
+    const long long tiles = (long long) ((p.M + FBM - 1) / FBM) * ((p.N + FBN - 1) / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
     return 2 * tiles <= num_cus ? 128 : 0;
 }
 
@@ -187,7 +201,7 @@ int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)
     q.split_k = 1;
     if (!gemm_large_tile_applicable(q)) return 0;
     const int       tm = p.tile_m == 128 ? 128 : FBM;
-    const long long tiles = (long long) ((p.M + tm - 1) / tm) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
+    const long long tiles = (long long) ((p.M + tm - 1) / tm) * ((p.N + FBN - 1) / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
     const int       nk = p.K * dt_bytes(p.dtype) / FBK;
     int             best = 1;
     // Splitting the reduction pays when the tiles leave most of the chip idle and the reduction is long: a slice costs a
@@ -216,7 +230,8 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
 {
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     const int       tm = p.tile_m == 128 ? 128 : FBM;
-    dim3            grid(((p.M + tm - 1) / tm) * (p.N / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    dim3            grid(((p.M + tm - 1) / tm) * ((p.N + FBN - 1) / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
+    if (large_tile_ragged(p)) return launch_gemm_large_tile_ragged(p, grid, s);
     if (tm == 128) return launch_gemm_large_tile_128(p, grid, s);
     if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return launch_conv_bf16(p, grid, s);

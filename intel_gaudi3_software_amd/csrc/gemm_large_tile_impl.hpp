@@ -124,7 +124,10 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // TM: rows of the output tile, 256 or 128 (128 for problems whose 256-row tiles would leave most of the chip idle; AMODE
 // 0, 1 and 3).  A wavefront then owns TM / 2 rows x 64 columns; an f-contiguous A stage is 32 k-rows of TM elements, one
 // request of 16 bytes per lane covers 2 (TM 256) or 4 (TM 128) of them.
-template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM>
+// RG ("ragged", AMODE 0 only): M is any count and N any multiple of 16: the loads of a partial tile are clamped to the
+// operand's last row / last 16-byte chunk and its stores are predicated.  A separate instantiation, so that the kernels for
+// whole tiles stay free of the clamps and predicates.
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
     static_assert(TM == 256 || (TM == 128 && AMODE != 2), "the 128-row tile is not instantiated for plain f-contiguous A");
@@ -135,13 +138,15 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     constexpr int  STAGE = A_BYTES + FBK * FBN;   // 32 KiB or 24 KiB
     constexpr int  NREQ = NUA + 2;                // requests per lane and stage
     constexpr bool GATHER = AMODE == 1;           // tap masks + uniform tap offsets
-    constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3; // the last row tile may be partial
+    static_assert(!RG || AMODE == 0, "partial column tiles are instantiated for plain k-contiguous A only");
+    constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3 || RG; // the last row tile may be partial
+    // (RG: the last column tile may be partial too; N is a multiple of 16, so a lane's 16 columns are all in or all out)
     constexpr bool A_KC = AMODE < 2;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
-    const int tiles_n = g.N / FBN, tiles_m = (g.M + TM - 1) / TM;
+    const int tiles_n = RG ? (g.N + FBN - 1) / FBN : g.N / FBN, tiles_m = (g.M + TM - 1) / TM;
     int       tm, tn;
     {
         const int b = blockIdx.x, T = tiles_m * tiles_n;
@@ -193,7 +198,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             if (u < NUA)
             {
                 const int r = (wave * NUA + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-                ga[u] = A + (size_t) (m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
+                ga[u] = A + (size_t) (RG ? min(m0 + r, g.M - 1) : m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
             }
         }
         if constexpr (AMODE == 2)
@@ -204,19 +209,19 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         if (B_KC)
         {
             const int r = t * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-            gb[u] = B + (size_t) (n0 + r) * ldb + c * 16 + (size_t) kt_begin * FBK;
+            gb[u] = B + (size_t) (RG ? min(n0 + r, g.N - 1) : n0 + r) * ldb + c * 16 + (size_t) kt_begin * FBK;
         }
         else if (GATHER && g.B.kind == VIEW_TAPPED)
             gb[u] = nullptr; // (tapped weights are k-contiguous: B_KC)
         else if (ES == 1)
         {
             const int k = t * 4 + (lane >> 4), p = lane & 15, cb = (p - 2 * (k & 7)) & 15;
-            gb[u] = B + (size_t) (k + kt_begin * FBK) * ldb + n0 + cb * 16;
+            gb[u] = B + (size_t) (k + kt_begin * FBK) * ldb + (RG ? min(n0 + cb * 16, g.N - 16) : n0 + cb * 16);
         }
         else
         {
             const int k = t * 2 + (lane >> 5), p = lane & 31, chunk = p ^ ((k & 3) << 1);
-            gb[u] = B + (size_t) (k + kt_begin * (FBK / 2)) * ldb + n0 * 2 + chunk * 16;
+            gb[u] = B + (size_t) (k + kt_begin * (FBK / 2)) * ldb + (RG ? min(n0 + chunk * 8, g.N - 8) : n0 + chunk * 8) * 2;
         }
     }
     // ---- GATHER: per-row tap masks and the running (tap, channel) position of the stage being requested ----------------
@@ -538,7 +543,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         if (col_exp)
         {
 #pragma unroll
-            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
+            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[RG ? min(n0 + wn * 64 + j * 32 + kg * 16 + c, g.N - 1) : n0 + wn * 64 + j * 32 + kg * 16 + c]);
         }
         if (relu)
         {
@@ -555,7 +560,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             {
                 float val[16];
                 gather(i, j, val);
-                if (!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
+                if ((!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) && (!RG || n0 + wn * 64 + j * 32 + kg * 16 < g.N))
+                    store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
             }
     };
     typedef float    e_v4f __attribute__((ext_vector_type(4)));
@@ -573,7 +579,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             for (int j = 0; j < 2; j++)
             {
                 e_v4f*     o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
-                const bool row_ok = !RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M;
+                const bool row_ok = (!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) && (!RG || n0 + wn * 64 + j * 32 + kg * 16 < g.N);
 #pragma unroll
                 for (int q = 0; q < 2; q++)
                 {
@@ -698,8 +704,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 {
                     float x = val[c];
                     if (has_alpha) x *= alpha;
-                    if (col_exp) x *= pow2_of(col_exp[n0 + wn * 64 + j * 32 + kg * 16 + c]);
-                    if (!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
+                    if (col_exp) x *= pow2_of(col_exp[RG ? min(n0 + wn * 64 + j * 32 + kg * 16 + c, g.N - 1) : n0 + wn * 64 + j * 32 + kg * 16 + c]);
+                    if ((!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) && (!RG || n0 + wn * 64 + j * 32 + kg * 16 < g.N)) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
                 }
             }
     }

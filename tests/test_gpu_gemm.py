@@ -348,3 +348,49 @@ def test_bf16_fast_kernel_every_k_position(calc, orc, b_kc):
                      MmeSimTensor([K, N] if b_kc else [N, K], 2, abi.BF16, tb), abi.OP_ABT if b_kc else abi.OP_AB)
     calc.synchronize()
     assert np.array_equal(out.cpu().numpy().reshape(M, N).astype(np.float64), want)
+
+
+# ---- the large-tile kernel on shapes that are not whole tiles: any M from 64 (A's rows along the tile's rows), N a multiple of 16
+RAGGED_FAST = [(300, 400, 384, (0, 0, 16), (1, 1, 1)), (77, 144, 2048, (0, 0, 0), (1, 1, 1)), (520, 272, 512, (0, 0, 0), (2, 1, 1))]
+
+
+@pytest.mark.parametrize("dtA,dtB,bA,bB", [(abi.FP8_143, abi.FP8_143, 7, 7), (abi.FP8_152, abi.FP8_143, 15, 11), (abi.BF16, abi.BF16, 0, 0)])
+@pytest.mark.parametrize("op", [abi.OP_AB, abi.OP_ABT])
+@pytest.mark.parametrize("M,N,K,pad,batch", RAGGED_FAST)
+def test_fast_kernel_partial_row_and_column_tiles(calc, orc, op, dtA, dtB, bA, bB, M, N, K, pad, batch):
+    """Loads of a partial tile stay inside the operands and its stores inside the output: the gap columns of a padded output
+    keep their zeros (the comparison covers them), a long reduction over few tiles is split over k."""
+    got, want = _run_both(calc, orc, op, M, N, K, dtA, dtB, bA, bB, 0, 0, batch=batch, bcast_b=batch != (1, 1, 1), seed=90 + op, device=True,
+                          pad=pad)
+    assert rel_frobenius(got, want) <= 1e-4
+    ld, nb = N + pad[2], int(np.prod(batch))
+    assert not got.reshape(M * nb, ld)[:, N:].any(), "gap columns were written"
+
+
+@pytest.mark.parametrize("out_dt,out_bias", [(abi.BF16, 0), (abi.FP8_143, 7), (abi.FP32, 0)])
+def test_fast_kernel_partial_tiles_fused_epilogue_bit_exact(calc, orc, out_dt, out_bias):
+    """Per-column scale exponents, descale, relu and the output cast on partial tiles: the fused output equals the oracle's
+    cast of the same kernel's fp32 accumulators, bit for bit."""
+    import torch
+    rng = np.random.default_rng(32)
+    M, N, K = 300, 400, 384
+    a = random_operand(rng, abi.FP8_143, M * K, orc, 7)
+    b = random_operand(rng, abi.FP8_152, N * K, orc, 15, scale=0.05)
+    col = rng.integers(-3, 4, N).astype(np.int32)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    acc = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    X = MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7)
+    W = MmeSimTensor([N, K], 2, abi.FP8_152, tb, 15)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, acc), X, W, abi.OP_AB)
+    td = {abi.BF16: torch.int16, abi.FP32: torch.float32}.get(out_dt, torch.uint8)
+    out = torch.zeros(M * N, dtype=td, device="cuda")
+    epi = Epilogue(scale_exp=-2, col_scale_exp=torch.from_numpy(col).cuda(), relu=True, clipFp=True)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, out_dt, out, out_bias), X, W, abi.OP_AB, epilogue=epi)
+    calc.synchronize()
+    acc_h = acc.cpu().numpy()
+    want = np.zeros(M * N, abi.DTYPE_NUMPY[out_dt] if out_dt != abi.FP32 else np.uint32)
+    assert orc.orc_cast_from_fp32(want.ctypes.data, out_dt, out_bias, 0, acc_h.ctypes.data, M * N, -2, col.ctypes.data, N, 1,
+                                  0, 1, 0, 0) == 0
+    got = out.cpu().numpy()
+    got = got.view(np.uint16) if out_dt == abi.BF16 else (got.view(np.uint32) if out_dt == abi.FP32 else got)
+    assert np.array_equal(got, want)
