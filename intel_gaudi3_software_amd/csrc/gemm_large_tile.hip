@@ -113,6 +113,7 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 hipError_t launch_gemm_large_tile_f16(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_f16.hip
 hipError_t launch_gemm_large_tile_128(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_128.hip
 hipError_t launch_gemm_large_tile_ragged(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged.hip
+hipError_t launch_gemm_large_tile_ragged_conv(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged_conv.hip
 
 // the shape is not made of whole tiles (the pixel rows of a convolution view do not count: every kernel handles those)
 static bool large_tile_ragged(const GemmProblem& p)
@@ -156,11 +157,12 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     if (!p.A.vec_ok || !p.B.vec_ok) return false;
     if (!p.A.k_contig && !two_byte) return false; // f-contiguous A: bf16 / fp16 only
     if (gather && p.A.pix_is_f && !p.A.k_contig) return false;
-    // whole tiles, except: the convolution views take any pixel count, and the GEMM forms with A k-contiguous have kernels for
-    // partial tiles (any M from 64, N a multiple of 16 from 128: a lane's 16 output columns are then all in or all out)
+    // whole tiles, except: the convolution views take any pixel count, and the convolutions and the GEMM forms with A
+    // k-contiguous have kernels for partial tiles (any M from 64, N a multiple of 16 from 128: a lane's 16 output columns
+    // are then all in or all out)
     if (large_tile_ragged(p))
     {
-        if (gather || !p.A.k_contig || p.M < 64 || p.N % 16 || p.N < FBN / 2) return false;
+        if ((!gather && !p.A.k_contig) || p.M < 64 || p.N % 16 || p.N < FBN / 2) return false;
     }
     if ((p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
     if (p.split_k > 1)
@@ -231,7 +233,7 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     const int       tm = p.tile_m == 128 ? 128 : FBM;
     dim3            grid(((p.M + tm - 1) / tm) * ((p.N + FBN - 1) / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
-    if (large_tile_ragged(p)) return launch_gemm_large_tile_ragged(p, grid, s);
+    if (large_tile_ragged(p)) return p.A.kind == VIEW_CONV ? launch_gemm_large_tile_ragged_conv(p, grid, s) : launch_gemm_large_tile_ragged(p, grid, s);
     if (tm == 128) return launch_gemm_large_tile_128(p, grid, s);
     if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return launch_conv_bf16(p, grid, s);

@@ -124,9 +124,9 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // TM: rows of the output tile, 256 or 128 (128 for problems whose 256-row tiles would leave most of the chip idle; AMODE
 // 0, 1 and 3).  A wavefront then owns TM / 2 rows x 64 columns; an f-contiguous A stage is 32 k-rows of TM elements, one
 // request of 16 bytes per lane covers 2 (TM 256) or 4 (TM 128) of them.
-// RG ("ragged", AMODE 0 only): M is any count and N any multiple of 16: the loads of a partial tile are clamped to the
-// operand's last row / last 16-byte chunk and its stores are predicated.  A separate instantiation, so that the kernels for
-// whole tiles stay free of the clamps and predicates.
+// RG ("ragged", not for AMODE 2): N is any multiple of 16 and, for AMODE 0, M any count (the convolution views take any pixel
+// count as they are): the loads of a partial tile are clamped to the operand's last row / last 16-byte chunk and its stores
+// are predicated.  A separate instantiation, so that the kernels for whole tiles stay free of the clamps and predicates.
 template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
@@ -138,7 +138,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     constexpr int  STAGE = A_BYTES + FBK * FBN;   // 32 KiB or 24 KiB
     constexpr int  NREQ = NUA + 2;                // requests per lane and stage
     constexpr bool GATHER = AMODE == 1;           // tap masks + uniform tap offsets
-    static_assert(!RG || AMODE == 0, "partial column tiles are instantiated for plain k-contiguous A only");
+    static_assert(!RG || AMODE != 2, "partial tiles are not instantiated for plain f-contiguous A");
     constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3 || RG; // the last row tile may be partial
     // (RG: the last column tile may be partial too; N is a multiple of 16, so a lane's 16 columns are all in or all out)
     constexpr bool A_KC = AMODE < 2;
@@ -285,7 +285,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             for (int u = 0; u < 2; u++)
             {
                 const int r = (wave * 2 + u) * 16 + (lane >> 2), p = lane & 3, c = p ^ ((r >> 2) & 3);
-                gb[u] = B + (size_t) (n0 + r) * ldb + c * 16;
+                gb[u] = B + (size_t) (RG ? min(n0 + r, g.N - 1) : n0 + r) * ldb + c * 16;
             }
         // first stage of this workgroup's k range
         const int k0 = kt_begin * stage_ch;

@@ -160,12 +160,15 @@ def test_conv_fwd_fast_path_special_values(calc, orc, relu, clip):
     assert np.array_equal(out.cpu().numpy().view(np.uint16), want16)
 
 
-# shapes that take the large-tile kernel with the gather on its load side: bf16, 256 output columns, channel counts that
-# are multiples of 32; ragged pixel counts, dilation, a strided forward pass, a 1 x 1 filter
+# shapes that take the large-tile kernel with the gather on its load side: 2-byte operands, at least 128 output columns (a
+# multiple of 16: the last column tile may be partial), channel counts that are multiples of 32; ragged pixel counts,
+# dilation, a strided forward pass, a 1 x 1 filter
 GATHER_CASES = [
     (256, 256, 9, 7, 1, 2, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),
     (64, 256, 11, 6, 1, 1, 3, 3, 1, (2, 2, 0), (1, 1, 1), (2, 2, 1), 2),
     (256, 256, 8, 8, 1, 1, 1, 1, 1, (0, 0, 0), (1, 1, 1), (1, 1, 1), 2),
+    (128, 192, 10, 7, 1, 2, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),   # fwd: 192 columns, dedx: 128 (partial column tiles)
+    (160, 400, 6, 5, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),    # fwd: two column tiles, the second partial
 ]
 
 
@@ -173,8 +176,8 @@ GATHER_CASES = [
 @pytest.mark.parametrize("op", [abi.OP_FWD, abi.OP_DEDX])
 @pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP16, 15), (abi.FP16, 11)])
 def test_conv_large_tile_gather_vs_oracle(calc, orc, case, op, dt, bias):
-    if op == abi.OP_DEDX and case[0] != 256:
-        pytest.skip("dedx has C output columns: only C = 256 takes the large-tile kernel")
+    if op == abi.OP_DEDX and case[0] < 128:
+        pytest.skip("dedx has C output columns: the large-tile kernel takes 128 or more")
     if case[6] == 1 and op == abi.OP_FWD:
         pass  # K * taps = 256 channels: 8 stages
     got, want = _run(calc, orc, case, dt, bias, op, device=True)
@@ -190,6 +193,7 @@ DEDW_CASES = [
     (64, 256, 16, 8, 1, 2, 3, 3, 1, (2, 2, 0), (1, 1, 1), (2, 2, 1), 2),     # M = 576: ragged row tile, three taps per tile
     (32, 256, 18, 17, 1, 1, 3, 3, 1, (0, 0, 0), (2, 2, 1), (1, 1, 1), 2),    # strided: 8 x 8 output pixels
     (256, 3840, 8, 8, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),
+    (96, 208, 16, 12, 1, 1, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),      # 208 output columns: a partial column tile
 ]
 
 
