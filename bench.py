@@ -261,7 +261,17 @@ def extra_measurements(calc, stream):
     res["conv_dedx_bf16_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_bf16_peak": fl / t / 1e12 / PEAK_TFLOPS["bf16"]}
     t = timed(lambda: calc.doConvolution(DW, XT, WT, YT, cp, abi.OP_DEDW), n=20)
     res["conv_dedw_bf16_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_bf16_peak": fl / t / 1e12 / PEAK_TFLOPS["bf16"]}
-    del XT, WT, YT, DX, DW
+    # the same layer with Gaudi fp8 operands (fp8_143 activations, bias 7; fp8_152 gradients, bias 15): fwd and dedx
+    q8 = lambda n, hi: torch.randint(0, hi, (n,), dtype=torch.uint8, device="cuda")
+    X8 = MmeSimTensor(xs, 5, abi.FP8_143, q8(int(np.prod(xs)), 0x60), 7)
+    W8 = MmeSimTensor(ws, 5, abi.FP8_143, q8(int(np.prod(ws)), 0x40), 7)
+    Y8 = MmeSimTensor(ys, 5, abi.FP8_152, q8(int(np.prod(ys)), 0x70), 15)
+    YO = MmeSimTensor(ys, 5, abi.FP32, torch.zeros(int(np.prod(ys)), dtype=torch.float32, device="cuda"))
+    t = timed(lambda: calc.doConvolution(YO, X8, W8, YO, cp, abi.OP_FWD), n=20)
+    res["conv_fwd_fp8_143_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
+    t = timed(lambda: calc.doConvolution(DX, X8, W8, Y8, cp, abi.OP_DEDX), n=20)
+    res["conv_dedx_fp8_152x143_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
+    del XT, WT, YT, DX, DW, X8, W8, Y8, YO
     # c5: batched mixed fp8: A fp8_143 (bias 7) [4096, 2048, 4] x B fp8_152 (bias 15) [14336, 4096, 1] (broadcast) -> fp8_143
     M5, K5, N5, b5 = 2048, 4096, 14336, 4
     qa = torch.randint(0, 0x78, (b5 * M5 * K5,), dtype=torch.uint8, device="cuda")

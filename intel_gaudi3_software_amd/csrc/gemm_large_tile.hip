@@ -112,6 +112,7 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 
 hipError_t launch_gemm_large_tile_f16(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_f16.hip
 hipError_t launch_gemm_large_tile_128(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_128.hip
+hipError_t launch_gemm_large_tile_conv_fp8(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_conv_fp8.hip
 hipError_t launch_gemm_large_tile_ragged(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged.hip
 hipError_t launch_gemm_large_tile_ragged_conv(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged_conv.hip
 
@@ -129,12 +130,14 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     const int  es = two_byte ? 2 : 1;
     const bool gather = p.A.kind == VIEW_CONV;
     const int  tm = p.tile_m == 128 ? 128 : FBM;
-    // the 128-row tile: 2-byte operands; A plain rows, the fwd / dedx gather, or dedw's pixels-along-k view
-    if (tm == 128 && (!two_byte || (!p.A.k_contig && !(gather && !p.A.pix_is_f)))) return false;
+    // the 128-row tile: 2-byte operands with A plain rows, the fwd / dedx gather or dedw's pixels-along-k view; fp8 operands
+    // with the fwd / dedx gather
+    if (tm == 128 && !two_byte && !(gather && p.A.pix_is_f)) return false;
+    if (tm == 128 && !p.A.k_contig && !(gather && !p.A.pix_is_f)) return false;
     if (gather)
     {
-        // bf16 / fp16, at most 32 taps, one problem per launch
-        if (!two_byte || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
+        // at most 32 taps, one problem per launch; fp8 for fwd / dedx only (dedw reads its operand through 16-bit transposes)
+        if ((!two_byte && !p.A.pix_is_f) || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
         if (p.batch[0] * p.batch[1] * p.batch[2] != 1) return false;
         if (p.A.pix_is_f)
         {
@@ -162,7 +165,7 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     // are then all in or all out)
     if (large_tile_ragged(p))
     {
-        if ((!gather && !p.A.k_contig) || p.M < 64 || p.N % 16 || p.N < FBN / 2) return false;
+        if ((!gather && !p.A.k_contig) || (gather && !two_byte) || p.M < 64 || p.N % 16 || p.N < FBN / 2) return false;
     }
     if ((p.K * es) % (2 * FBK) || p.K * es < 6 * FBK) return false;
     if (p.split_k > 1)
@@ -234,9 +237,10 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
     const int       tm = p.tile_m == 128 ? 128 : FBM;
     dim3            grid(((p.M + tm - 1) / tm) * ((p.N + FBN - 1) / FBN), (unsigned) nb, p.split_k > 1 ? p.split_k : 1);
     if (large_tile_ragged(p)) return p.A.kind == VIEW_CONV ? launch_gemm_large_tile_ragged_conv(p, grid, s) : launch_gemm_large_tile_ragged(p, grid, s);
+    if (tm == 128 && p.dtype != DT_BF16 && p.dtype != DT_FP16) return launch_gemm_large_tile_conv_fp8(p, grid, s);
     if (tm == 128) return launch_gemm_large_tile_128(p, grid, s);
     if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
-    if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return launch_conv_bf16(p, grid, s);
+    if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return p.dtype == DT_BF16 ? launch_conv_bf16(p, grid, s) : launch_gemm_large_tile_conv_fp8(p, grid, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {

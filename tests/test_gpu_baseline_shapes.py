@@ -157,19 +157,22 @@ def test_large_tile_kernel_both_tile_heights(calc, orc, dt):
             assert rel_frobenius(got[r0:r0 + 64].ravel(), want) <= 1e-4, (M, r0)
 
 
-def test_conv_gather_with_256_row_tiles(calc, orc):
+@pytest.mark.parametrize("dt,dt_y,bias,bias_y", [(abi.BF16, abi.BF16, 0, 0), (abi.FP8_143, abi.FP8_152, 7, 15)])
+def test_conv_gather_with_256_row_tiles(calc, orc, dt, dt_y, bias, bias_y):
     """A 3 x 3 forward convolution and dedx with enough pixels for more than 128 tiles of 256 rows (43 images of 28 x 28, 256
-    channels: 132 tiles), so that the gather runs on the 256-row kernel; first and last image against the oracle."""
+    channels: 132 tiles), so that the gather runs on the 256-row kernel (bf16, and fp8 with the gradient in the other fp8
+    flavour); first and last image against the oracle."""
     import torch
+    from helpers import random_operand
     rng = np.random.default_rng(4)
     B, H, W, Cc, Kk = 43, 28, 28, 256, 256
     xs, ws, ys = [Cc, W, H, 1, B], [Kk, Cc, 3, 3, 1], [Kk, W, H, 1, B]
-    x = to_bf16_bits(rng.standard_normal(int(np.prod(xs))).astype(np.float32))
-    w = to_bf16_bits((rng.standard_normal(int(np.prod(ws))) * 0.02).astype(np.float32))
-    dy = to_bf16_bits(rng.standard_normal(int(np.prod(ys))).astype(np.float32))
+    x = random_operand(rng, dt, int(np.prod(xs)), orc, bias)
+    w = random_operand(rng, dt, int(np.prod(ws)), orc, bias, scale=0.05)
+    dy = random_operand(rng, dt_y, int(np.prod(ys)), orc, bias_y)
     cp = ConvolutionParams(2, [1, 1, 0, 0])
     p = abi.make_conv_params(2, (1, 1, 0), (1, 1, 1), (1, 1, 1))
-    X, Wt, DY = MmeSimTensor(xs, 5, abi.BF16, _dev(x)), MmeSimTensor(ws, 5, abi.BF16, _dev(w)), MmeSimTensor(ys, 5, abi.BF16, _dev(dy))
+    X, Wt, DY = MmeSimTensor(xs, 5, dt, _dev(x), bias), MmeSimTensor(ws, 5, dt, _dev(w), bias), MmeSimTensor(ys, 5, dt_y, _dev(dy), bias_y)
     gy = torch.zeros(int(np.prod(ys)), dtype=torch.float32, device="cuda")
     gdx = torch.zeros(int(np.prod(xs)), dtype=torch.float32, device="cuda")
     out_y = MmeSimTensor(ys, 5, abi.FP32, gy)
@@ -181,8 +184,8 @@ def test_conv_gather_with_256_row_tiles(calc, orc):
     for b in (0, B - 1):
         xb, yb = np.ascontiguousarray(x[b * per_x:(b + 1) * per_x]), np.ascontiguousarray(dy[b * per_y:(b + 1) * per_y])
         want_y, want_dx = np.zeros(per_y, np.float32), np.zeros(per_x, np.float32)
-        dxb, dwd = desc(xb, [Cc, W, H, 1, 1], abi.BF16), desc(w, ws, abi.BF16)
-        doy, dox, dyb = desc(want_y, [Kk, W, H, 1, 1], abi.FP32), desc(want_dx, [Cc, W, H, 1, 1], abi.FP32), desc(yb, [Kk, W, H, 1, 1], abi.BF16)
+        dxb, dwd = desc(xb, [Cc, W, H, 1, 1], dt, bias), desc(w, ws, dt, bias)
+        doy, dox, dyb = desc(want_y, [Kk, W, H, 1, 1], abi.FP32), desc(want_dx, [Cc, W, H, 1, 1], abi.FP32), desc(yb, [Kk, W, H, 1, 1], dt_y, bias_y)
         assert orc.orc_convolution(A(doy), A(dxb), A(dwd), A(doy), A(p), abi.OP_FWD, 0) == 0
         assert orc.orc_convolution(A(dox), A(dox), A(dwd), A(dyb), A(p), abi.OP_DEDX, 0) == 0
         assert rel_frobenius(yg[b], want_y) <= 1e-4 and rel_frobenius(dxg[b], want_dx) <= 1e-4

@@ -174,7 +174,7 @@ GATHER_CASES = [
 
 @pytest.mark.parametrize("case", GATHER_CASES)
 @pytest.mark.parametrize("op", [abi.OP_FWD, abi.OP_DEDX])
-@pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP16, 15), (abi.FP16, 11)])
+@pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP16, 15), (abi.FP16, 11), (abi.FP8_143, 7), (abi.FP8_143, 11), (abi.FP8_152, 15)])
 def test_conv_large_tile_gather_vs_oracle(calc, orc, case, op, dt, bias):
     if op == abi.OP_DEDX and case[0] < 128:
         pytest.skip("dedx has C output columns: the large-tile kernel takes 128 or more")
