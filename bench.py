@@ -271,6 +271,8 @@ def extra_measurements(calc, stream):
     res["conv_fwd_fp8_143_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
     t = timed(lambda: calc.doConvolution(DX, X8, W8, Y8, cp, abi.OP_DEDX), n=20)
     res["conv_dedx_fp8_152x143_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
+    t = timed(lambda: calc.doConvolution(DW, X8, W8, Y8, cp, abi.OP_DEDW), n=20)
+    res["conv_dedw_fp8_143x152_n32_28x28_c256_k256_3x3"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
     del XT, WT, YT, DX, DW, X8, W8, Y8, YO
     # c5: batched mixed fp8: A fp8_143 (bias 7) [4096, 2048, 4] x B fp8_152 (bias 15) [14336, 4096, 1] (broadcast) -> fp8_143
     M5, K5, N5, b5 = 2048, 4096, 14336, 4
@@ -284,6 +286,14 @@ def extra_measurements(calc, stream):
     fl = 2.0 * b5 * M5 * N5 * K5
     t = timed(lambda: calc.doBatchGemm(Y5, A5, B5, abi.OP_AB, epilogue=e5), n=10, warm=2)
     res["bgemm_fp8_143x152_4x2048x14336x4096_fp8_out"] = {"seconds": t, "TFLOP/s": fl / t / 1e12, "frac_fp8_peak": fl / t / 1e12 / PEAK_TFLOPS["fp8"]}
+    # fp8 GEMM with A stored K x M ("atb": A read through transposing LDS loads)
+    nt = 4096
+    qt = lambda: torch.randint(0, 0x60, (nt * nt,), dtype=torch.uint8, device="cuda")
+    AT, BT = MmeSimTensor([nt, nt], 2, abi.FP8_143, qt(), 7), MmeSimTensor([nt, nt], 2, abi.FP8_143, qt(), 7)
+    YT8 = MmeSimTensor([nt, nt], 2, abi.FP32, torch.zeros(nt * nt, dtype=torch.float32, device="cuda"))
+    t = timed(lambda: calc.doBatchGemm(YT8, AT, BT, abi.OP_ATB), n=20)
+    res["gemm_fp8_143_atb_4096x4096x4096_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * nt ** 3 / t / 1e12, "frac_fp8_peak": 2.0 * nt ** 3 / t / 1e12 / PEAK_TFLOPS["fp8"]}
+    del AT, BT, YT8
     # the fp16 flavours last: their work spaces (two bf16 copies of both operands) are the largest allocations of the run
     n4 = 4096
     h16 = lambda: torch.randn(n4 * n4, device="cuda").to(torch.float16).view(torch.int16)

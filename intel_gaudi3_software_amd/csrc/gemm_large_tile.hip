@@ -113,6 +113,7 @@ hipError_t launch_fmt(const GemmProblem& p, dim3 grid, hipStream_t s)
 hipError_t launch_gemm_large_tile_f16(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_f16.hip
 hipError_t launch_gemm_large_tile_128(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_128.hip
 hipError_t launch_gemm_large_tile_conv_fp8(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_conv_fp8.hip
+hipError_t launch_gemm_large_tile_fp8_at(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_fp8_at.hip
 hipError_t launch_gemm_large_tile_ragged(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged.hip
 hipError_t launch_gemm_large_tile_ragged_conv(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged_conv.hip
 
@@ -136,8 +137,8 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     if (tm == 128 && !p.A.k_contig && !(gather && !p.A.pix_is_f)) return false;
     if (gather)
     {
-        // at most 32 taps, one problem per launch; fp8 for fwd / dedx only (dedw reads its operand through 16-bit transposes)
-        if ((!two_byte && !p.A.pix_is_f) || p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
+        // at most 32 taps, one problem per launch
+        if (p.A.ktap[0] * p.A.ktap[1] * p.A.ktap[2] > 32) return false;
         if (p.batch[0] * p.batch[1] * p.batch[2] != 1) return false;
         if (p.A.pix_is_f)
         {
@@ -152,13 +153,12 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
         else
         {
             // dedw: 16-byte chunks of channels inside one tap, dY plain with its channels contiguous
-            if (p.A.gather_y || p.A.nch % 8 || p.B.kind != VIEW_PLAIN || p.B.k_contig) return false;
+            if (p.A.gather_y || p.A.nch % (16 / es) || p.B.kind != VIEW_PLAIN || p.B.k_contig) return false;
         }
     }
     else if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN)
         return false;
     if (!p.A.vec_ok || !p.B.vec_ok) return false;
-    if (!p.A.k_contig && !two_byte) return false; // f-contiguous A: bf16 / fp16 only
     if (gather && p.A.pix_is_f && !p.A.k_contig) return false;
     // whole tiles, except: the convolution views take any pixel count, and the convolutions and the GEMM forms with A
     // k-contiguous have kernels for partial tiles (any M from 64, N a multiple of 16 from 128: a lane's 16 output columns
@@ -242,6 +242,7 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
     if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return p.dtype == DT_BF16 ? launch_conv_bf16(p, grid, s) : launch_gemm_large_tile_conv_fp8(p, grid, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
+    if (!p.A.k_contig) return launch_gemm_large_tile_fp8_at(p, grid, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {
         case 0: return launch_fmt<0>(p, grid, s);

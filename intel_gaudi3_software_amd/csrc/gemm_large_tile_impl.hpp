@@ -98,6 +98,21 @@ __device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int
     f.a[i] = u.v;
 }
 
+// fp8, A stored f-contiguous: the stage layout and reads of an n-contiguous fp8 B (64 k-rows x 256 bytes), over the
+// wavefront's 128 rows = 8 chunks of 16
+__device__ __forceinline__ void read_a_tr8(Frags& f, int i, const char* st, int wm, int lane)
+{
+    const int q = lane >> 4, cb = wm * 8 + i * 2 + (q & 1), g = q >> 1, rr = (lane & 15) >> 1, h = lane & 1;
+    v2i       t[4];
+#pragma unroll
+    for (int tt = 0; tt < 4; tt++)
+    {
+        const int k = g * 32 + 8 * tt + rr;
+        t[tt] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS3 v2i*) (st + fb_pos(k, cb) * 16 + h * 8));
+    }
+    f.a[i] = v8i {t[0].x, t[0].y, t[1].x, t[1].y, t[2].x, t[2].y, t[3].x, t[3].y};
+}
+
 // B stored k-contiguous (the "abt" form): same layout and reads as A
 __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int wn, int lane)
 {
@@ -131,6 +146,7 @@ template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = fals
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
     static_assert(TM == 256 || (TM == 128 && AMODE != 2), "the 128-row tile is not instantiated for plain f-contiguous A");
+    static_assert(TM == 256 || ES == 2 || AMODE < 2, "fp8 operands that are contiguous along the tile's rows: 256-row tiles only");
     constexpr int  WR = TM / 2;                   // rows per wavefront
     constexpr int  NI = WR / 32;                  // A fragments (32-row blocks) per wavefront
     constexpr int  NUA = TM / 128;                // A requests per lane and stage (16 rows x 64 bytes per wavefront and request)
@@ -201,10 +217,15 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 ga[u] = A + (size_t) (RG ? min(m0 + r, g.M - 1) : m0 + r) * lda + c * 16 + (size_t) kt_begin * FBK;
             }
         }
-        if constexpr (AMODE == 2)
+        if constexpr (AMODE == 2 && ES == 2)
         {
             const int k = t * 2 + (lane >> 5), p = lane & 31, chunk = p ^ ((k & 3) << 1);
             ga[u] = A + (size_t) (k + kt_begin * (FBK / 2)) * lda + m0 * 2 + chunk * 16;
+        }
+        if constexpr (AMODE == 2 && ES == 1)
+        {
+            const int k = t * 4 + (lane >> 4), p = lane & 15, cb = (p - 2 * (k & 7)) & 15;
+            ga[u] = A + (size_t) (k + kt_begin * FBK) * lda + m0 + cb * 16;
         }
         if (B_KC)
         {
@@ -309,14 +330,16 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         for (int u = 0; u < 2; u++)
         {
             if (u >= NUA) break;
-            constexpr int RPQ = 512 / TM; // k-rows per request
-            const int     kr = (wave * NUA + u) * RPQ + lane / (64 / RPQ), chunk = (lane & (64 / RPQ - 1)) ^ ((kr & 3) << 1);
-            const int     f = m0 + chunk * 8, tap = f / g.A.nch;
-            w_ch[u] = f < g.M ? (long long) (f - tap * g.A.nch) * 2 : -1;
+            constexpr int RPQ = ES == 1 ? 4 : 512 / TM; // k-rows per request
+            const int     kr = (wave * NUA + u) * RPQ + lane / (64 / RPQ);
+            // 16-byte chunk of the row that this lane fetches (the swizzles of the two stage layouts)
+            const int chunk = ES == 1 ? ((lane & 15) - 2 * (kr & 7)) & 15 : (lane & (64 / RPQ - 1)) ^ ((kr & 3) << 1);
+            const int f = m0 + chunk * (16 / ES), tap = f / g.A.nch;
+            w_ch[u] = f < g.M ? (long long) (f - tap * g.A.nch) * ES : -1;
             w_t[u][0] = tap % g.A.ktap[0];
             w_t[u][1] = (tap / g.A.ktap[0]) % g.A.ktap[1];
             w_t[u][2] = tap / (g.A.ktap[0] * g.A.ktap[1]);
-            const PixelPos pp = decode_pixel(g.A, kt_begin * (FBK / 2) + kr);
+            const PixelPos pp = decode_pixel(g.A, kt_begin * (FBK / ES) + kr);
 #pragma unroll
             for (int d = 0; d < 4; d++) w_pc[u][d] = pp.c[d];
         }
@@ -333,12 +356,12 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             {
                 const int pos = w_pc[u][d] * g.A.cstride[d] + (d < 3 ? w_t[u][d] * g.A.dil[d] : 0) - g.A.pad[d];
                 ok = ok && pos >= 0 && pos < g.A.src[d];
-                off += (long long) pos * g.A.src_stride[d] * 2;
+                off += (long long) pos * g.A.src_stride[d] * ES;
             }
             const uint8_t* src = ok ? A + off : (const uint8_t*) gf_zero_page;
             dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
-            // next stage: 32 pixels further
-            int carry = 32;
+            // next stage: 32 (2-byte elements) or 64 (fp8) pixels further
+            int carry = FBK / ES;
 #pragma unroll
             for (int d = 0; d < 3; d++)
             {
@@ -400,6 +423,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
     {
         if constexpr (A_KC) read_a(fr, i, st, wm * WR, lane);
+        else if constexpr (ES == 1)
+            read_a_tr8(fr, i, st, wm, lane);
         else
             read_a_tr16<TM>(fr, i, st, wm, lane);
     };

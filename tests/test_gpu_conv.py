@@ -194,11 +194,12 @@ DEDW_CASES = [
     (32, 256, 18, 17, 1, 1, 3, 3, 1, (0, 0, 0), (2, 2, 1), (1, 1, 1), 2),    # strided: 8 x 8 output pixels
     (256, 3840, 8, 8, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),
     (96, 208, 16, 12, 1, 1, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),      # 208 output columns: a partial column tile
+    (64, 256, 16, 8, 1, 3, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2),       # 384 pixels: enough for the fp8 kernel's k-stages
 ]
 
 
 @pytest.mark.parametrize("case", DEDW_CASES)
-@pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP16, 15)])
+@pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP16, 15), (abi.FP8_143, 7), (abi.FP8_152, 15)])
 def test_conv_large_tile_dedw_vs_oracle(calc, orc, case, dt, bias):
     got, want = _run(calc, orc, case, dt, bias, abi.OP_DEDW, device=True)
     assert rel_frobenius(got, want) <= TOL[dt]

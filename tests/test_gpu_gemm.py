@@ -195,19 +195,20 @@ def test_gemm_linearity_large(calc, orc):
 # ---- the large-aligned fp8 kernel (256 x 256 tiles, LDS DMA ring, transposed LDS reads) ---------------------------------
 @pytest.mark.parametrize("dtA,dtB,bA,bB", [(abi.FP8_143, abi.FP8_143, 7, 7), (abi.FP8_143, abi.FP8_152, 7, 15),
                                            (abi.FP8_152, abi.FP8_143, 15, 11), (abi.FP8_152, abi.FP8_152, 20, 15)])
-@pytest.mark.parametrize("op", [abi.OP_AB, abi.OP_ABT])
+@pytest.mark.parametrize("op", OPS)
 def test_fp8_fast_kernel_vs_oracle(calc, orc, op, dtA, dtB, bA, bB):
     """Shapes that take the fast path (M, N multiples of 256, K multiple of 128 and >= 384), every fp8 flavour pair,
-    both B layouts, batch of 2 with B broadcast; fp32 accumulators against the oracle."""
+    all four layouts, batch of 2 with B broadcast; fp32 accumulators against the oracle."""
     got, want = _run_both(calc, orc, op, 256, 512, 384, dtA, dtB, bA, bB, 0, 0, batch=(2, 1, 1), bcast_b=True, seed=50 + op,
                           device=True)
     assert rel_frobenius(got, want) <= 1e-2
     assert rel_frobenius(got, want) <= 1e-4  # the reference's truncating tree itself sits ~1e-5 from the exact sums
 
 
-def test_fp8_fast_kernel_every_k_position(calc, orc):
+@pytest.mark.parametrize("a_transposed", [False, True])
+def test_fp8_fast_kernel_every_k_position(calc, orc, a_transposed):
     """One-hot operands walk a single product through every k position and every tile coordinate: catches any
-    fragment / swizzle / transposed-read mix-up that random data could average out."""
+    fragment / swizzle / transposed-read mix-up that random data could average out.  A as M x K rows or stored K x M."""
     import torch
     M, N, K = 256, 256, 512
     one = 0x38  # 1.0 in fp8_143 bias 7
@@ -219,10 +220,11 @@ def test_fp8_fast_kernel_every_k_position(calc, orc):
         a[perm_m[k % M], k] = one
         b[k, (k * 7 + 3) % N] = 0x40 if k % 2 else one   # 2.0 / 1.0
     want = (a == one).astype(np.float64) @ np.where(b == 0x40, 2.0, (b == one) * 1.0)
-    ta, tb = torch.from_numpy(a.ravel()).cuda(), torch.from_numpy(b.ravel()).cuda()
+    a_stored = np.ascontiguousarray(a.T) if a_transposed else a
+    ta, tb = torch.from_numpy(a_stored.ravel()).cuda(), torch.from_numpy(b.ravel()).cuda()
     out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
-    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7),
-                     MmeSimTensor([N, K], 2, abi.FP8_143, tb, 7), abi.OP_AB)
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([M, K] if a_transposed else [K, M], 2, abi.FP8_143, ta, 7),
+                     MmeSimTensor([N, K], 2, abi.FP8_143, tb, 7), abi.OP_ATB if a_transposed else abi.OP_AB)
     calc.synchronize()
     assert np.array_equal(out.cpu().numpy().reshape(M, N).astype(np.float64), want)
 
