@@ -131,9 +131,8 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     const int  es = two_byte ? 2 : 1;
     const bool gather = p.A.kind == VIEW_CONV;
     const int  tm = p.tile_m == 128 ? 128 : FBM;
-    // the 128-row tile: 2-byte operands with A plain rows, the fwd / dedx gather or dedw's pixels-along-k view; fp8 operands
-    // with the fwd / dedx gather
-    if (tm == 128 && !two_byte && !(gather && p.A.pix_is_f)) return false;
+    // the 128-row tile: A plain rows or the fwd / dedx gather; 2-byte operands also with dedw's pixels-along-k view
+    if (tm == 128 && !two_byte && !p.A.k_contig) return false;
     if (tm == 128 && !p.A.k_contig && !(gather && !p.A.pix_is_f)) return false;
     if (gather)
     {

@@ -131,29 +131,31 @@ def test_c5_batched_mixed_fp8_gemm_full_size(calc, orc):
         assert np.count_nonzero(want & 0x7F) > rows * N // 2  # the slab is not a field of zeros
 
 
-@pytest.mark.parametrize("dt", [abi.BF16, abi.FP16])
-def test_large_tile_kernel_both_tile_heights(calc, orc, dt):
+TILE_HEIGHT_TYPES = [(abi.BF16, abi.BF16, 0, 0), (abi.FP16, abi.FP16, 15, 15), (abi.FP8_143, abi.FP8_143, 7, 7), (abi.FP8_143, abi.FP8_152, 7, 15),
+                     (abi.FP8_152, abi.FP8_143, 15, 11), (abi.FP8_152, abi.FP8_152, 20, 15)]
+
+
+@pytest.mark.parametrize("dtA,dtB,bA,bB", TILE_HEIGHT_TYPES)
+@pytest.mark.parametrize("op", [abi.OP_AB, abi.OP_ABT])
+def test_large_tile_kernel_both_tile_heights(calc, orc, op, dtA, dtB, bA, bB):
     """The large-tile kernel picks 128-row tiles when 256-row tiles would occupy at most half of the compute units, else
-    256-row ones.  A bf16 / fp16 GEMM with 144 tiles of 256 x 256 (the 256-row kernel) and one with M = 384 (the 128-row
-    kernel; M is not a multiple of 256): slabs of rows against the oracle."""
+    256-row ones.  A GEMM with 144 tiles of 256 x 256 (the 256-row kernel) and one with M = 384 (the 128-row kernel; M is
+    not a multiple of 256), bf16, fp16 and every pair of fp8 flavours, both layouts of B: slabs of rows against the oracle."""
     import torch
+    from helpers import random_operand
     rng = np.random.default_rng(3)
-    for (M, N, K) in [(3072, 3072, 320), (384, 512, 448)]:
-        if dt == abi.BF16:
-            a, b = (to_bf16_bits(rng.standard_normal(n).astype(np.float32)) for n in (M * K, N * K))
-        else:
-            a, b = (rng.standard_normal(n).astype(np.float16).view(np.uint16) for n in (M * K, N * K))
-        bias = 15 if dt == abi.FP16 else 0
+    for (M, N, K) in [(3072, 3072, 384), (384, 512, 512)]:
+        a, b = random_operand(rng, dtA, M * K, orc, bA), random_operand(rng, dtB, N * K, orc, bB)
+        bsz = [K, N] if op == abi.OP_ABT else [N, K]
         out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
-        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, dt, _dev(a), bias), MmeSimTensor([K, N], 2, dt, _dev(b), bias),
-                         abi.OP_ABT)
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, dtA, _dev(a), bA), MmeSimTensor(bsz, 2, dtB, _dev(b), bB), op)
         calc.synchronize()
         got = out.cpu().numpy().reshape(M, N)
         for r0 in (0, M // 2 - 32, M - 64):
             slab = np.ascontiguousarray(a.reshape(M, K)[r0:r0 + 64])
             want = np.zeros(64 * N, np.float32)
-            da, db, do = desc(slab, [K, 64], dt, bias), desc(b, [K, N], dt, bias), desc(want, [N, 64], abi.FP32)
-            assert orc.orc_batch_gemm(A(do), A(da), A(db), abi.OP_ABT) == 0
+            da, db, do = desc(slab, [K, 64], dtA, bA), desc(b, bsz, dtB, bB), desc(want, [N, 64], abi.FP32)
+            assert orc.orc_batch_gemm(A(do), A(da), A(db), op) == 0
             assert rel_frobenius(got[r0:r0 + 64].ravel(), want) <= 1e-4, (M, r0)
 
 
