@@ -308,7 +308,13 @@ def extra_measurements(calc, stream):
     # 2 M N K, the fraction prices the four bf16 products per multiply-add that the matrix cores execute
     res["gemm_ufp16_4096x4096x4096_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n4 ** 3 / t / 1e12,
                                                  "frac_bf16_peak_of_issued_products": 4 * 2.0 * n4 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
-    del AH, BH, AU, BU, YH
+    # fp32 operands: three bf16 parts per value, six cross products on the bf16 matrix cores
+    f32 = lambda: torch.randn(n4 * n4, device="cuda")
+    AF, BF = MmeSimTensor([n4, n4], 2, abi.FP32, f32()), MmeSimTensor([n4, n4], 2, abi.FP32, f32())
+    t = timed(lambda: calc.doBatchGemm(YH, AF, BF, abi.OP_ABT), n=10, warm=2)
+    res["gemm_fp32_4096x4096x4096_fp32_out"] = {"seconds": t, "TFLOP/s": 2.0 * n4 ** 3 / t / 1e12, "frac_fp32_peak": 2.0 * n4 ** 3 / t / 1e12 / PEAK_TFLOPS["fp32"],
+                                                "frac_bf16_peak_of_issued_products": 6 * 2.0 * n4 ** 3 / t / 1e12 / PEAK_TFLOPS["bf16"]}
+    del AH, BH, AU, BU, YH, AF, BF
     nc = 1 << 28
     xc = torch.randn(nc, device="cuda")
     oc = torch.zeros(nc, dtype=torch.int16, device="cuda")

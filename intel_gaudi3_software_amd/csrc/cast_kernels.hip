@@ -653,26 +653,32 @@ hipError_t launch_round_to_tf32(void* out, const void* in, size_t n, int clip, i
 // otherwise; batch dimensions the source broadcasts (stride 0) have extent 1 in the copy.  A value that is not finite
 // cannot be split (inf * 0 appears among the partial products): it stores `epoch` into *flag and the caller's predicated
 // launches take the fp32 path instead.  V elements per lane along the contiguous index (8 with 16-byte accesses, or 1).
+// fp32 operands (24 significant bits) take three parts, value = hi + mid + lo of 8 bits each, and six K-blocks: A as
+// [hi | hi | mid | hi | lo | mid], B as [hi | mid | hi | lo | hi | mid]; the three products left out (mid lo, lo mid, lo lo)
+// are below 2^-23 of hi hi, the rounding step of the fp32 accumulation itself.
 template<int DT, int V>
 __global__ __launch_bounds__(CAST_THREADS) void split_bf16_kernel(uint16_t* __restrict__ out, const void* __restrict__ in, SplitBf16Args a)
 {
     const long long C = a.k_contig ? a.K : a.F, O = a.k_contig ? a.F : a.K, groups = C / V;
     const long long total = groups * O * a.e[0] * a.e[1] * a.e[2];
-    const long long part = a.k_contig ? (long long) a.K : (long long) a.K * a.F; // elements between the four parts
+    const long long part = a.k_contig ? (long long) a.K : (long long) a.K * a.F; // elements between the K-blocks
     const int       hi_part1 = a.is_b ? 2 : 1, lo_part0 = a.is_b ? 1 : 2;          // hi -> parts 0 and hi_part1, lo -> lo_part0 and 3
+    constexpr int   NB = DT == DT_FP32 ? 6 : 4;                                    // K-blocks
+    // three parts: which part (0 hi, 1 mid, 2 lo) each of the six K-blocks holds
+    const int       p3[6] = {0, a.is_b ? 1 : 0, a.is_b ? 0 : 1, a.is_b ? 2 : 0, a.is_b ? 0 : 2, 1};
     bool            special = false;
     for (long long t = (long long) blockIdx.x * CAST_THREADS + threadIdx.x; t < total; t += (long long) gridDim.x * CAST_THREADS)
     {
         const long long cg = t % groups, r = t / groups, o = r % O;
         long long       b = r / O;
         const long long f = a.k_contig ? o : cg * V, k = a.k_contig ? cg * V : o;
-        const long long dst = a.k_contig ? (b * a.F + f) * 4 * a.K + k : (b * 4 * a.K + k) * a.F + f;
+        const long long dst = a.k_contig ? (b * a.F + f) * NB * a.K + k : (b * NB * a.K + k) * a.F + f;
         const int       b0 = (int) (b % a.e[0]);
         b /= a.e[0];
         const int       b1 = (int) (b % a.e[1]), b2 = (int) (b / a.e[1]);
         const long long src = b0 * a.bs[0] + b1 * a.bs[1] + b2 * a.bs[2] + f * a.sf + k * a.sk;
         uint32_t        raw[V];
-        if constexpr (V == 8 && DT == DT_TF32)
+        if constexpr (V == 8 && (DT == DT_TF32 || DT == DT_FP32))
         {
             const v4u x = *(const v4u*) ((const uint32_t*) in + src), y = *(const v4u*) ((const uint32_t*) in + src + 4);
             raw[0] = x.x, raw[1] = x.y, raw[2] = x.z, raw[3] = x.w, raw[4] = y.x, raw[5] = y.y, raw[6] = y.z, raw[7] = y.w;
@@ -683,24 +689,55 @@ __global__ __launch_bounds__(CAST_THREADS) void split_bf16_kernel(uint16_t* __re
             raw[0] = x.x & 0xFFFFu, raw[1] = x.x >> 16, raw[2] = x.y & 0xFFFFu, raw[3] = x.y >> 16;
             raw[4] = x.z & 0xFFFFu, raw[5] = x.z >> 16, raw[6] = x.w & 0xFFFFu, raw[7] = x.w >> 16;
         }
-        else if constexpr (DT == DT_TF32)
+        else if constexpr (DT == DT_TF32 || DT == DT_FP32)
             raw[0] = ((const uint32_t*) in)[src];
         else
             raw[0] = ((const uint16_t*) in)[src];
-        uint32_t hi[V], lo[V];
+        uint32_t hi[V], lo[V], mid[V];
 #pragma unroll
         for (int j = 0; j < V; j++)
         {
             uint32_t u;
             if constexpr (DT == DT_TF32) u = fp32_to_tf32(raw[j], a.clip, a.clip_inf_in);
+            else if constexpr (DT == DT_FP32)
+                u = raw[j];
             else
                 u = f2u(decode1<DT>(raw[j], a.bias, a.mode));
             special = special || ((u & 0x7F800000u) == 0x7F800000u);
             const uint32_t h = u & 0xFFFF0000u;
             hi[j] = h >> 16;
-            lo[j] = f2u(u2f(u) - u2f(h)) >> 16;
+            const float rest = u2f(u) - u2f(h);
+            if constexpr (DT == DT_FP32)
+            {
+                const uint32_t m = f2u(rest) & 0xFFFF0000u;
+                mid[j] = m >> 16;
+                lo[j] = f2u(rest - u2f(m)) >> 16;
+            }
+            else
+            {
+                mid[j] = 0;
+                lo[j] = f2u(rest) >> 16;
+            }
         }
-        if constexpr (V == 8)
+        if constexpr (DT == DT_FP32)
+        {
+            // six K-blocks
+#pragma unroll
+            for (int blk = 0; blk < 6; blk++)
+            {
+                const int which = p3[blk];
+                if constexpr (V == 8)
+                {
+                    uint32_t w[8];
+#pragma unroll
+                    for (int j = 0; j < 8; j++) w[j] = which == 0 ? hi[j] : (which == 1 ? mid[j] : lo[j]);
+                    *(v4u*) (out + dst + blk * part) = v4u {w[0] | (w[1] << 16), w[2] | (w[3] << 16), w[4] | (w[5] << 16), w[6] | (w[7] << 16)};
+                }
+                else
+                    out[dst + blk * part] = (uint16_t) (which == 0 ? hi[0] : (which == 1 ? mid[0] : lo[0]));
+            }
+        }
+        else if constexpr (V == 8)
         {
             const v4u h4 = {hi[0] | (hi[1] << 16), hi[2] | (hi[3] << 16), hi[4] | (hi[5] << 16), hi[6] | (hi[7] << 16)};
             const v4u l4 = {lo[0] | (lo[1] << 16), lo[2] | (lo[3] << 16), lo[4] | (lo[5] << 16), lo[6] | (lo[7] << 16)};
@@ -744,6 +781,7 @@ hipError_t launch_split_bf16(uint16_t* out, const void* in, int dtype, const Spl
         case DT_FP16: return launch_split_dt<DT_FP16>(out, in, a, s);
         case DT_UFP16: return launch_split_dt<DT_UFP16>(out, in, a, s);
         case DT_TF32: return launch_split_dt<DT_TF32>(out, in, a, s);
+        case DT_FP32: return launch_split_dt<DT_FP32>(out, in, a, s);
         default: return hipErrorInvalidValue;
     }
 }

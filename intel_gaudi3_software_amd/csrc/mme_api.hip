@@ -300,7 +300,9 @@ int plan_launch(mme_hip_handle h, GemmProblem& g)
 // combination (unsigned fp16 with its 6-bit exponent, exponent-all-ones codes that are finite, tf32) is contracted here:
 //  - plain GEMMs of some size: each operand is written as two bf16 parts that add up to its exact value and the bf16 kernels
 //    contract the 4 K long rows (split_bf16_kernel); operands that hold inf or NaN raise a device flag, which skips that
-//    contraction and lets the fp32 one below run instead, so the call never waits for the device;
+//    contraction and lets the fp32 one below run instead, so the call never waits for the device.  fp32 operands take the
+//    same route with three bf16 parts and six of the nine cross products (6 K long rows; the fall-back then reads the
+//    operands themselves);
 //  - everything else: fp32 words holding the operands' exact values (tf32: the rounded ones), in the operands' own layout,
 //    contracted by the fp32 instantiation.
 int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, const mme_hip_tensor* tb, const void* a_base, const void* b_base,
@@ -313,9 +315,16 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
         return fold_alpha(h, g.epi, (15 - (int) ta->fp_bias) + (15 - (int) tb->fp_bias));
     }
     done = true;
+    const bool      fp32_in = ta->dtype == MME_HIP_FP32;
+    const int       kblocks = fp32_in ? 6 : 4; // K-blocks of the split copies
     const long long nbatch = (long long) g.batch[0] * g.batch[1] * g.batch[2];
     const bool      two_part = g.A.kind == VIEW_PLAIN && g.B.kind == VIEW_PLAIN && (long long) g.M * g.N * g.K * nbatch >= (1ll << 26) &&
-                          g.K <= (1 << 28);
+                          g.K <= (1 << 27);
+    if (fp32_in && !two_part)
+    {
+        done = false; // plain fp32 contraction: the caller launches it
+        return MME_HIP_OK;
+    }
     const size_t na = span_elements(ta), nb = span_elements(tb);
     const size_t na_pad = (na + 3) & ~(size_t) 3;
     size_t       part_elems[2] = {0, 0};
@@ -325,7 +334,7 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
     if (two_part)
         for (int i = 0; i < 2; i++)
         {
-            part_elems[i] = (size_t) free_extent[i] * g.K * 4;
+            part_elems[i] = (size_t) free_extent[i] * g.K * kblocks;
             for (int d = 0; d < 3; d++)
             {
                 eff[i][d] = view[i]->batch_stride[d] ? g.batch[d] : 1;
@@ -333,10 +342,11 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
             }
             part_elems[i] = (part_elems[i] + 7) & ~(size_t) 7;
         }
-    HIP_TRY(h, h->decode_ws.reserve((na_pad + nb + 4) * 4 + (part_elems[0] + part_elems[1]) * 2));
+    const size_t fp32_copies = fp32_in ? 0 : na_pad + ((nb + 3) & ~(size_t) 3);
+    HIP_TRY(h, h->decode_ws.reserve((fp32_copies + 4) * 4 + (part_elems[0] + part_elems[1]) * 2));
     float*    da = (float*) h->decode_ws.p;
     float*    db = da + na_pad;
-    uint16_t* parts = (uint16_t*) (db + ((nb + 3) & ~(size_t) 3));
+    uint16_t* parts = (uint16_t*) ((float*) h->decode_ws.p + fp32_copies);
     const mme_hip_tensor* t[2] = {ta, tb};
     const void*           src[2] = {a_base, b_base};
     uint32_t*             flag = nullptr;
@@ -364,7 +374,7 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
             a.clip_inf_in = h->operand_clip_inf_in;
             a.flag = flag;
             a.epoch = epoch;
-            long long bstride[3], run = (long long) a.F * a.K * 4;
+            long long bstride[3], run = (long long) a.F * a.K * kblocks;
             for (int d = 0; d < 3; d++)
             {
                 a.e[d] = (int) eff[i][d];
@@ -373,16 +383,16 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
                 run *= eff[i][d];
             }
             HIP_TRY(h, launch_split_bf16(dst, src[i], t[i]->dtype, a, h->stream));
-            if (a.k_contig) set_plain_view(*v2[i], dst, 4ll * a.K, 1, true, 2, 4 * a.K, bstride);
+            if (a.k_contig) set_plain_view(*v2[i], dst, (long long) kblocks * a.K, 1, true, 2, kblocks * a.K, bstride);
             else
                 set_plain_view(*v2[i], dst, 1, a.F, false, 2, a.F, bstride);
             dst += part_elems[i];
         }
         g2.dtype = DT_BF16;
-        g2.K = 4 * g.K;
+        g2.K = kblocks * g.K;
     }
     // the fp32 contraction: the only one, or the one that runs when an operand holds inf / NaN
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 2 && !fp32_in; i++)
     {
         float* d = i ? db : da;
         if (t[i]->dtype == MME_HIP_TF32)
@@ -392,8 +402,11 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
                                            flag, epoch));
     }
     g.dtype = DT_FP32;
-    g.A.base = (const char*) da;
-    g.B.base = (const char*) db;
+    if (!fp32_in)
+    {
+        g.A.base = (const char*) da;
+        g.B.base = (const char*) db;
+    }
     g.skip_flag = flag;
     g.skip_epoch = epoch;
     g.skip_if = 0; // runs when the flag holds this call's epoch
@@ -418,7 +431,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
 {
     g.skip_flag = nullptr;
     g.skip_if = 0;
-    if (is_fp16(g.dtype) || g.dtype == MME_HIP_TF32)
+    if (is_fp16(g.dtype) || g.dtype == MME_HIP_TF32 || g.dtype == MME_HIP_FP32)
     {
         bool done = false;
         if (int rc = run_half_contraction(h, g, ta, tb, a_base, b_base, done)) return rc;

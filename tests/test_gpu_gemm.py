@@ -396,3 +396,76 @@ def test_fast_kernel_partial_tiles_fused_epilogue_bit_exact(calc, orc, out_dt, o
     got = out.cpu().numpy()
     got = got.view(np.uint16) if out_dt == abi.BF16 else (got.view(np.uint32) if out_dt == abi.FP32 else got)
     assert np.array_equal(got, want)
+
+
+# ---- fp32 operands on the bf16 matrix cores: three bf16 parts per value, six cross products (plain GEMMs from 2^26 multiply-adds)
+@pytest.mark.parametrize("op", OPS)
+def test_fp32_three_part_path_vs_oracle_and_float64(calc, orc, op):
+    """An aligned shape (the large-tile bf16 kernel over 6 K) and a ragged, batched one (the general kernel): within 1e-4 of
+    the oracle like every fast kernel, and within 2e-6 of the float64 product, i.e. at the level of fp32 accumulation: the
+    three cross products that are left out do not show."""
+    for (M, N, K, batch) in [(256, 256, 1024, (1, 1, 1)), (200, 136, 1237, (2, 1, 1))]:
+        got, want = _run_both(calc, orc, op, M, N, K, abi.FP32, abi.FP32, 0, 0, 0, 0, batch=batch, bcast_b=batch != (1, 1, 1), seed=120 + op,
+                              device=True)
+        assert rel_frobenius(got, want) <= 1e-4, (M, N, K)
+        rng = np.random.default_rng(120 + op)          # the operands _run_both drew
+        asz, bsz = _shapes(op, M, N, K)
+        nb = int(np.prod(batch))
+        a = random_operand(rng, abi.FP32, asz[0] * asz[1] * nb, orc).astype(np.float64).reshape(nb, asz[1], asz[0])
+        b = random_operand(rng, abi.FP32, bsz[0] * bsz[1], orc).astype(np.float64).reshape(bsz[1], bsz[0])
+        am = a.transpose(0, 2, 1) if op in (abi.OP_ATB, abi.OP_ATBT) else a      # (nb, M, K)
+        bm = b.T if op in (abi.OP_ABT, abi.OP_ATBT) else b                        # (K, N)
+        exact = (am @ bm).ravel()
+        assert rel_frobenius(got, exact) <= 2e-6, (M, N, K)
+
+
+def test_fp32_three_part_path_keeps_all_24_bits(calc, orc):
+    """One-hot operands with full 24-bit significands against powers of two: every product is exact, so the output has to
+    reproduce the operand bit for bit at every k position of the six K-blocks."""
+    import torch
+    M, N, K = 256, 256, 1024
+    rng = np.random.default_rng(8)
+    a = np.zeros((M, K), np.float32)
+    b = np.zeros((K, N), np.float32)
+    perm_m = rng.permutation(M)
+    vals = (1.0 + rng.integers(1, 1 << 23, K) * 2.0 ** -23).astype(np.float32) * np.where(rng.random(K) < 0.5, -1, 1).astype(np.float32)
+    for k in range(K):
+        a[perm_m[k % M], k] = vals[k]
+        b[k, (k * 11 + 2 + 64 * (k // M)) % N] = 0.5 if k % 2 else 4.0
+    want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, abi.FP32, torch.from_numpy(a.ravel()).cuda()),
+                     MmeSimTensor([N, K], 2, abi.FP32, torch.from_numpy(b.ravel()).cuda()), abi.OP_AB)
+    calc.synchronize()
+    assert np.array_equal(out.cpu().numpy().reshape(M, N), want)
+    # and the other way round: full significands in B
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, abi.FP32, torch.from_numpy((a != 0).astype(np.float32).ravel() * 2).cuda()),
+                     MmeSimTensor([N, K], 2, abi.FP32, torch.from_numpy((np.where(b != 0, 1, 0) * vals[:, None]).astype(np.float32).ravel()).cuda()), abi.OP_AB)
+    calc.synchronize()
+    want2 = ((a != 0).astype(np.float64) * 2) @ (np.where(b != 0, 1, 0) * vals[:, None].astype(np.float64))
+    assert np.array_equal(out.cpu().numpy().reshape(M, N).astype(np.float64), want2)
+
+
+def test_fp32_three_part_path_steps_aside_for_inf_and_nan(calc, orc):
+    """inf and NaN among fp32 operands: the contraction runs on the fp32 instantiation instead (decided on the device)."""
+    M, N, K = 256, 256, 1024
+    rng = np.random.default_rng(11)
+    a = rng.standard_normal(M * K).astype(np.float32)
+    b = rng.standard_normal(N * K).astype(np.float32)
+    a.reshape(M, K)[3, 5], a.reshape(M, K)[7, 9] = np.inf, np.nan
+    b.reshape(K, N)[5, 2] = 0.0
+    import torch
+    out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, abi.FP32, torch.from_numpy(a).cuda()),
+                     MmeSimTensor([N, K], 2, abi.FP32, torch.from_numpy(b).cuda()), abi.OP_AB)
+    calc.synchronize()
+    got = out.cpu().numpy().reshape(M, N)
+    want = np.zeros(M * N, np.float32)
+    assert orc.orc_batch_gemm(A(desc(want, [N, M, 1, 1, 1], abi.FP32)), A(desc(a, [K, M, 1, 1, 1], abi.FP32)), A(desc(b, [N, K, 1, 1, 1], abi.FP32)),
+                              abi.OP_AB) == 0
+    want = want.reshape(M, N)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.isnan(want[3, 2]) and np.isnan(want[7]).all()
+    inf = np.isinf(want)
+    assert inf.any() and np.array_equal(got[inf], want[inf])
+    fin = np.isfinite(want)
+    assert rel_frobenius(got[fin], want[fin]) <= 1e-4
