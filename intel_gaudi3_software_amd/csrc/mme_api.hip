@@ -318,7 +318,7 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
     const bool      fp32_in = ta->dtype == MME_HIP_FP32;
     const int       kblocks = fp32_in ? 6 : 4; // K-blocks of the split copies
     const long long nbatch = (long long) g.batch[0] * g.batch[1] * g.batch[2];
-    const bool      two_part = g.A.kind == VIEW_PLAIN && g.B.kind == VIEW_PLAIN && (long long) g.M * g.N * g.K * nbatch >= (1ll << 26) &&
+    bool            two_part = g.A.kind == VIEW_PLAIN && g.B.kind == VIEW_PLAIN && (long long) g.M * g.N * g.K * nbatch >= (1ll << 26) &&
                           g.K <= (1 << 27);
     if (fp32_in && !two_part)
     {
@@ -342,6 +342,17 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
             }
             part_elems[i] = (part_elems[i] + 7) & ~(size_t) 7;
         }
+    if (two_part && (part_elems[0] + part_elems[1]) * 2 > ((size_t) 16 << 30))
+    {
+        // the split copies would need more than 16 GiB of work space: contract the operands as they are
+        if (fp32_in)
+        {
+            done = false;
+            return MME_HIP_OK;
+        }
+        two_part = false;
+        part_elems[0] = part_elems[1] = 0;
+    }
     const size_t fp32_copies = fp32_in ? 0 : na_pad + ((nb + 3) & ~(size_t) 3);
     HIP_TRY(h, h->decode_ws.reserve((fp32_copies + 4) * 4 + (part_elems[0] + part_elems[1]) * 2));
     float*    da = (float*) h->decode_ws.p;
