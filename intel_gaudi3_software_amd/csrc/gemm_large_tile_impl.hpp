@@ -548,7 +548,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     // element offset of this lane's first value in block (0, 0): row m0 + wm * WR + lane % 32, column n0 + wn * 64 + 16 kg
     const long long lane_elem = c_off + (long long) (m0 + wm * WR + (lane & 31)) * ldc + n0 + wn * 64 + kg * 16;
     // block (i, j) -> the lane's 16 values after the power-of-two factors and relu
-    auto gather = [&](int i, int j, float (&val)[16]) __attribute__((always_inline))
+    auto gather = [&](int i, int j, float (&val)[16], auto raw_c) __attribute__((always_inline))
     {
 #pragma unroll
         for (int q = 0; q < 2; q++)
@@ -560,6 +560,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 val[8 * q + r] = __uint_as_float(sw[0]);
                 val[8 * q + 4 + r] = __uint_as_float(sw[1]);
             }
+        if constexpr (decltype(raw_c)::value) return;
         if (has_alpha)
         {
 #pragma unroll
@@ -576,71 +577,80 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             for (int c = 0; c < 16; c++) val[c] = relu_ref(val[c]);
         }
     };
-    auto walk = [&](auto store) __attribute__((always_inline))
-    {
-#pragma unroll
-        for (int i = 0; i < NI; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-            {
-                float val[16];
-                gather(i, j, val);
-                if ((!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) && (!RG || n0 + wn * 64 + j * 32 + kg * 16 < g.N))
-                    store(lane_elem + (long long) (i * 32) * ldc + j * 32, val);
-            }
-    };
     typedef float    e_v4f __attribute__((ext_vector_type(4)));
     typedef uint32_t e_v4u __attribute__((ext_vector_type(4)));
     typedef float    e_v2f __attribute__((ext_vector_type(2)));
     typedef __bf16   e_v2bf __attribute__((ext_vector_type(2)));
-    if (g.split_k > 1)
+    // Converted values pass through LDS on their way out (the ring is idle by now): a lane holds 16 columns of one row, and
+    // stored from there a 128-byte line of the output would arrive as four to eight separate pieces.  Each wavefront stages
+    // one 32-row block of its 64 columns (16-byte chunks XOR-swizzled by row, conflict-free both ways) and stores it back
+    // with consecutive lanes on consecutive chunks of a row: whole lines per request.
+    auto walk_to = [&](auto esz_c, auto raw_c, uint8_t* outb, long long pitch, auto pack) __attribute__((always_inline))
     {
-        // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
-        float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N +
-                    (long long) (m0 + wm * WR + (lane & 31)) * g.N + n0 + wn * 64 + kg * 16;
+        constexpr int ESZ = decltype(esz_c)::value; // bytes per output element = 16-byte chunks per lane and block
+        constexpr int RB = 64 * ESZ, CPR = RB / 16, NRD = RB / 32;
+        char*         stg = lds + wave * (32 * RB);
+        const int     row = lane & 31, swz = (row * CPR / 16) & (CPR - 1);
+        constexpr bool RAW = decltype(raw_c)::value; // partial sums of a k-slice: no factors, no relu
+        __syncthreads(); // the slowest wavefront has taken its last fragments out of the ring
 #pragma unroll
         for (int i = 0; i < NI; i++)
+        {
 #pragma unroll
             for (int j = 0; j < 2; j++)
             {
-                e_v4f*     o = (e_v4f*) (ws + (long long) (i * 32) * g.N + j * 32);
-                const bool row_ok = (!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) && (!RG || n0 + wn * 64 + j * 32 + kg * 16 < g.N);
+                float    val[16];
+                uint32_t pk[4 * ESZ];
+                gather(i, j, val, raw_c);
+                pack(val, pk);
 #pragma unroll
-                for (int q = 0; q < 2; q++)
-                {
-                    float lo4[4], hi4[4];
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                    {
-                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint((float) acc[i][j][4 * q + r]),
-                                                                         __float_as_uint((float) acc[i][j][8 + 4 * q + r]), false, false);
-                        lo4[r] = __uint_as_float(sw[0]);
-                        hi4[r] = __uint_as_float(sw[1]);
-                    }
-                    if (row_ok)
-                    {
-                        o[2 * q] = e_v4f {lo4[0], lo4[1], lo4[2], lo4[3]};
-                        o[2 * q + 1] = e_v4f {hi4[0], hi4[1], hi4[2], hi4[3]};
-                    }
-                }
+                for (int h = 0; h < ESZ; h++)
+                    *(e_v4u*) (stg + row * RB + ((((j * 2 + kg) * ESZ + h) ^ swz) << 4)) = e_v4u {pk[4 * h], pk[4 * h + 1], pk[4 * h + 2], pk[4 * h + 3]};
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int r = 0; r < NRD; r++)
+            {
+                const int   q = r * 64 + lane, rr = q / CPR, lc = q % CPR;
+                const e_v4u v = *(const e_v4u*) (stg + rr * RB + ((lc ^ ((rr * CPR / 16) & (CPR - 1))) << 4));
+                if ((!RAGGED_M || m0 + wm * WR + i * 32 + rr < g.M) && (!RG || n0 + wn * 64 + lc * (16 / ESZ) < g.N))
+                    *(e_v4u*) (outb + (long long) (i * 32 + rr) * pitch + lc * 16) = v;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+        (void) RAW;
+    };
+    auto walk = [&](auto esz_c, auto pack) __attribute__((always_inline))
+    {
+        constexpr int ESZ = decltype(esz_c)::value;
+        walk_to(esz_c, std::false_type(), (uint8_t*) g.epi.out + (c_off + (long long) (m0 + wm * WR) * ldc + n0 + wn * 64) * ESZ, ldc * ESZ, pack);
+    };
+    if (g.split_k > 1)
+    {
+        // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
+        float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N + (long long) (m0 + wm * WR) * g.N + n0 + wn * 64;
+        walk_to(std::integral_constant<int, 4>(), std::true_type(), (uint8_t*) ws, (long long) g.N * 4, [&](const float (&val)[16], uint32_t (&pk)[16]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int c = 0; c < 16; c++) pk[c] = __float_as_uint(val[c]);
+        });
     }
     else if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
-        walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
-            e_v4f* o = (e_v4f*) ((float*) g.epi.out + idx);
+        walk(std::integral_constant<int, 4>(), [&](const float (&val)[16], uint32_t (&pk)[16]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int c = 0; c < 4; c++) o[c] = e_v4f {val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3]};
+            for (int c = 0; c < 16; c++) pk[c] = __float_as_uint(val[c]);
         });
     else if (dt == DT_BF16 && g.epi.fast_cast)
         // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN (checked over
         // all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x| over
         // the lane's 16 values detects them and the block is then converted element by element
-        walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
+        walk(std::integral_constant<int, 2>(), [&](const float (&val)[16], uint32_t (&pk)[8]) __attribute__((always_inline)) {
             float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
             const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
-            uint32_t   pk[8];
             if (__builtin_amdgcn_ballot_w64(special) == 0)
             {
 #pragma unroll
@@ -656,23 +666,19 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 for (int c = 0; c < 8; c++)
                     pk[c] = fp32_to_bf16_rne(f2u(val[2 * c]), cp.clip_fp, cp.clip_inf_in) | (fp32_to_bf16_rne(f2u(val[2 * c + 1]), cp.clip_fp, cp.clip_inf_in) << 16);
             }
-            e_v4u* o = (e_v4u*) ((uint16_t*) g.epi.out + idx);
-            o[0] = e_v4u {pk[0], pk[1], pk[2], pk[3]};
-            o[1] = e_v4u {pk[4], pk[5], pk[6], pk[7]};
         });
     else if ((dt == DT_FP8_143 || dt == DT_FP8_152) && g.epi.fast_cast)
     {
         auto fp8_store = [&](auto m_c) __attribute__((always_inline))
         {
             constexpr int MAN = decltype(m_c)::value;
-            walk([&](long long idx, const float (&val)[16]) __attribute__((always_inline)) {
+            walk(std::integral_constant<int, 1>(), [&](const float (&val)[16], uint32_t (&pk)[4]) __attribute__((always_inline)) {
                 // the hardware converter equals the reference's conversion on finite inputs; a block that holds inf or
                 // NaN (sum of magnitudes not finite) takes the exact converter
                 float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
                 const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) <= 0x1.fffffep+127f);
-                uint32_t   pk[4];
                 if (__builtin_amdgcn_ballot_w64(special) == 0)
                 {
 #pragma unroll
@@ -689,7 +695,6 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                             pk[c] |= (fp32_to_fp8_rne_mode0<MAN>(f2u(val[4 * c + e]), cp.exp_bias, cp.clip_fp, cp.clip_inf_in) & 0xFFu) << (8 * e);
                     }
                 }
-                *(e_v4u*) ((uint8_t*) g.epi.out + idx) = e_v4u {pk[0], pk[1], pk[2], pk[3]};
             });
         };
         if (dt == DT_FP8_143) fp8_store(std::integral_constant<int, 3>());
