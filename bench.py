@@ -30,7 +30,7 @@ METRIC = "TFLOP/s & % fp8/bf16 MFMA peak (GEMM, conv); cast GB/s vs HBM peak; 1 
 
 # HBM bytes per launch of the fp8 GEMM kernel on this workload, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
 # profiles/gemm_fp8_fast_kernel_4096x4096x4096_hbm_traffic.txt (96.3 MiB fetched + 32.1 MiB written; 64 MiB algorithmic)
-GEMM_TRAFFIC_BYTES = 134.7e6
+GEMM_TRAFFIC_BYTES = 134.6e6
 
 
 def pow2_scale_exp(absmax, fmax):
