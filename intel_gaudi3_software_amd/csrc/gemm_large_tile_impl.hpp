@@ -616,7 +616,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 const int   q = r * 64 + lane, rr = q / CPR, lc = q % CPR;
                 const e_v4u v = *(const e_v4u*) (stg + rr * RB + ((lc ^ ((rr * CPR / 16) & (CPR - 1))) << 4));
                 if ((!RAGGED_M || m0 + wm * WR + i * 32 + rr < g.M) && (!RG || n0 + wn * 64 + lc * (16 / ESZ) < g.N))
-                    *(e_v4u*) (outb + (long long) (i * 32 + rr) * pitch + lc * 16) = v;
+                    __builtin_nontemporal_store(v, (e_v4u*) (outb + (long long) (i * 32 + rr) * pitch + lc * 16));
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
