@@ -123,6 +123,29 @@ __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int w
 
 #define FENCE __builtin_amdgcn_sched_barrier(0)
 
+// The problem description is read in place from the kernarg segment, field by field where the code needs it: every 64-byte
+// line touched for the first time (tile set-up, gather set-up, epilogue) would be a miss of its own, one memory latency
+// each, in series.  One scalar load per line up front takes all those misses at once.
+__device__ __forceinline__ void warm_kernargs(KARG GemmProblem& g)
+{
+    static_assert(sizeof(GemmProblem) <= 640, "one load per 64-byte line of the problem description");
+    uint32_t t0, t1, t2, t3, t4, t5, t6, t7, t8, t9;
+    asm volatile("s_load_dword %0, %10, 0x0\n\t"
+                 "s_load_dword %1, %10, 0x40\n\t"
+                 "s_load_dword %2, %10, 0x80\n\t"
+                 "s_load_dword %3, %10, 0xc0\n\t"
+                 "s_load_dword %4, %10, 0x100\n\t"
+                 "s_load_dword %5, %10, 0x140\n\t"
+                 "s_load_dword %6, %10, 0x180\n\t"
+                 "s_load_dword %7, %10, 0x1c0\n\t"
+                 "s_load_dword %8, %10, 0x200\n\t"
+                 "s_load_dword %9, %10, 0x240\n\t"
+                 "s_waitcnt lgkmcnt(0)"
+                 : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9)
+                 : "s"(&g)
+                 : "memory");
+}
+
 // ES = 1: fp8 (FMT selects e4m3 / e5m2 per operand), ES = 2: bf16 (FMT 0) or IEEE half (FMT 1).  Everything up to the matrix-core instruction is
 // byte-based and shared: a stage is 64 bytes of k per row for both.
 // GATHER: A is a convolution view with pixels along f (im2col addressing of mme/mme_reference/im2col.cpp:134-172 for the
@@ -159,6 +182,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     // (RG: the last column tile may be partial too; N is a multiple of 16, so a lane's 16 columns are all in or all out)
     constexpr bool A_KC = AMODE < 2;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
+    warm_kernargs(g);
     if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
