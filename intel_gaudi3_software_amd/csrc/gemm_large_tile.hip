@@ -116,6 +116,8 @@ hipError_t launch_gemm_large_tile_conv_fp8(const GemmProblem& p, dim3 grid, hipS
 hipError_t launch_gemm_large_tile_fp8_at(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_fp8_at.hip
 hipError_t launch_gemm_large_tile_ragged(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged.hip
 hipError_t launch_gemm_large_tile_ragged_conv(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged_conv.hip
+bool       gemm_large_tile_persistent_applicable(const GemmProblem& p);                      // gemm_large_tile_persistent.hip
+hipError_t launch_gemm_large_tile_persistent(const GemmProblem& p, hipStream_t s);
 
 // the shape is not made of whole tiles (the pixel rows of a convolution view do not count: every kernel handles those)
 static bool large_tile_ragged(const GemmProblem& p)
@@ -242,6 +244,7 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return p.dtype == DT_BF16 ? launch_conv_bf16(p, grid, s) : launch_gemm_large_tile_conv_fp8(p, grid, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     if (!p.A.k_contig) return launch_gemm_large_tile_fp8_at(p, grid, s);
+    if (gemm_large_tile_persistent_applicable(p)) return launch_gemm_large_tile_persistent(p, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {
         case 0: return launch_fmt<0>(p, grid, s);

@@ -165,9 +165,14 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // RG ("ragged", not for AMODE 2): N is any multiple of 16 and, for AMODE 0, M any count (the convolution views take any pixel
 // count as they are): the loads of a partial tile are clamped to the operand's last row / last 16-byte chunk and its stores
 // are predicated.  A separate instantiation, so that the kernels for whole tiles stay free of the clamps and predicates.
-template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false>
+// PERSIST (AMODE 0, whole 256-row tiles, 1- or 2-byte fused outputs, no split-k; gridDim = (256, 1, 1) and 160 KiB of LDS):
+// a workgroup walks over tiles id, id + 256, ... of all batch elements.  Once the last fragments of a tile have left the
+// ring, the first four stages of the next tile are requested, and the epilogue of the finished tile (which stages its
+// stores in the 32 KiB of LDS behind the ring) runs while they arrive: pipeline fill and epilogue overlap.
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
+    static_assert(!PERSIST || (AMODE == 0 && TM == FBM && !RG), "the persistent schedule: plain k-contiguous A, whole 256-row tiles");
     static_assert(TM == 256 || (TM == 128 && AMODE != 2), "the 128-row tile is not instantiated for plain f-contiguous A");
     static_assert(TM == 256 || ES == 2 || AMODE < 2, "fp8 operands that are contiguous along the tile's rows: 256-row tiles only");
     constexpr int  WR = TM / 2;                   // rows per wavefront
@@ -187,32 +192,46 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
     const int tiles_n = RG ? (g.N + FBN - 1) / FBN : g.N / FBN, tiles_m = (g.M + TM - 1) / TM;
-    int       tm, tn;
+    const int tiles_total = tiles_m * tiles_n;
+    int       m0 = 0, n0 = 0, b0 = 0, b1 = 0, b2 = 0;
+    const long long lda = (A_KC ? g.A.stride_f : g.A.stride_k) * ES; // bytes between rows of the staged A tile
+    const long long ldb = (B_KC ? g.B.stride_f : g.B.stride_k) * ES;
+    const uint8_t*  A = nullptr;
+    const uint8_t*  B = nullptr;
+    // tile L of the walk (each XCD owns a compact 8 x 4 block of tiles at a time) and batch element bz -> m0, n0, A, B
+    auto locate = [&](int L, int bz) __attribute__((always_inline))
     {
-        const int b = blockIdx.x, T = tiles_m * tiles_n;
+        int tm, tn;
         if ((tiles_m % 8 == 0) && (tiles_n % 4 == 0))
         {
-            const int L = (b & 7) * (T >> 3) + (b >> 3), Bx = L >> 5, w = L & 31, nbn = tiles_n >> 2;
+            const int Bx = L >> 5, w = L & 31, nbn = tiles_n >> 2;
             tm = (Bx / nbn) * 8 + (w >> 2);
             tn = (Bx % nbn) * 4 + (w & 3);
         }
         else
         {
-            tm = b / tiles_n;
-            tn = b % tiles_n;
+            tm = L / tiles_n;
+            tn = L % tiles_n;
         }
-    }
-    int       bz = blockIdx.y;
-    const int b0 = bz % g.batch[0];
-    bz /= g.batch[0];
-    const int       b1 = bz % g.batch[1], b2 = bz / g.batch[1];
-    const long long a_off = b0 * g.A.batch_stride[0] + b1 * g.A.batch_stride[1] + b2 * g.A.batch_stride[2];
-    const long long b_off = b0 * g.B.batch_stride[0] + b1 * g.B.batch_stride[1] + b2 * g.B.batch_stride[2];
-    const int       m0 = tm * TM, n0 = tn * FBN;
-    const long long lda = (A_KC ? g.A.stride_f : g.A.stride_k) * ES; // bytes between rows of the staged A tile
-    const long long ldb = (B_KC ? g.B.stride_f : g.B.stride_k) * ES;
-    const uint8_t*  A = (const uint8_t*) g.A.base + a_off * ES;
-    const uint8_t*  B = (const uint8_t*) g.B.base + b_off * ES;
+        b0 = bz % g.batch[0];
+        bz /= g.batch[0];
+        b1 = bz % g.batch[1];
+        b2 = bz / g.batch[1];
+        const long long a_off = b0 * g.A.batch_stride[0] + b1 * g.A.batch_stride[1] + b2 * g.A.batch_stride[2];
+        const long long b_off = b0 * g.B.batch_stride[0] + b1 * g.B.batch_stride[1] + b2 * g.B.batch_stride[2];
+        m0 = tm * TM;
+        n0 = tn * FBN;
+        A = (const uint8_t*) g.A.base + a_off * ES;
+        B = (const uint8_t*) g.B.base + b_off * ES;
+    };
+    // workgroup ids are dealt round-robin to the 8 XCDs
+    const int walk_first = PERSIST ? (int) ((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : 0;
+    const int walk_total = PERSIST ? tiles_total * g.batch[0] * g.batch[1] * g.batch[2] : 0;
+    if constexpr (PERSIST) locate(walk_first % tiles_total, walk_first / tiles_total);
+    else if ((tiles_m % 8 == 0) && (tiles_n % 4 == 0))
+        locate((blockIdx.x & 7) * (tiles_total >> 3) + (blockIdx.x >> 3), blockIdx.y);
+    else
+        locate(blockIdx.x, blockIdx.y);
     const uint32_t  lds_base = (uint32_t) (uintptr_t) lds;
 
     v16f acc[NI][2];
@@ -228,6 +247,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     // per-lane global pointers of this wavefront's 2 + 2 request slots (they advance by one stage per step)
     const uint8_t* ga[2];
     const uint8_t* gb[2];
+    auto setup_ptrs = [&]() __attribute__((always_inline))
+    {
 #pragma unroll
     for (int u = 0; u < 2; u++)
     {
@@ -269,6 +290,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             gb[u] = B + (size_t) (k + kt_begin * (FBK / 2)) * ldb + (RG ? min(n0 + chunk * 8, g.N - 8) : n0 + chunk * 8) * 2;
         }
     }
+    };
+    setup_ptrs();
     // ---- GATHER: per-row tap masks and the running (tap, channel) position of the stage being requested ----------------
     uint32_t  tap_ok[2] = {0, 0};      // bit t: tap t of this lane's row (request slot u) reads inside the source tensor
     int       g_tap = 0, g_ch = 0;     // uniform: tap and first channel of the next stage to request
@@ -432,17 +455,34 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 
     // all four slots of the ring are requested up front: a slot is free again as soon as its stage has been copied into
     // fragment registers, which happens one step before the stage is multiplied
-    for (int t = 0; t < FNST; t++)
+    auto issue_prologue = [&]() __attribute__((always_inline))
     {
-#pragma unroll
-        for (int u = 0; u < 2; u++)
+        for (int t = 0; t < FNST; t++)
         {
-            if (u < NUA) issue_a(u, t, t);
-            issue_b(u, t, t);
+#pragma unroll
+            for (int u = 0; u < 2; u++)
+            {
+                if (u < NUA) issue_a(u, t, t);
+                issue_b(u, t, t);
+            }
         }
-    }
+    };
+    issue_prologue();
+    for (int walk_it = 0;;) // (one pass unless PERSIST)
+    {
     // s_waitcnt immediate (gfx9): vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * NREQ)); // three stages may still be in flight: stage 0 has landed
+    if (!PERSIST || walk_it == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * NREQ)); // three stages may still be in flight: stage 0 has landed
+    else
+    {
+        // a later tile: its four stages were requested before the previous tile's epilogue, whose stores share the counter
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+        for (int i = 0; i < NI; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    }
     __syncthreads();
     auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
     {
@@ -559,6 +599,30 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     // every lane with 16 consecutive columns of one row, stored 16 bytes at a time.  The output-type dispatch sits
     // outside the unrolled block walk so that the accumulators stay in registers.
     const long long c_off = b0 * g.epi.batch_stride[0] + b1 * g.epi.batch_stride[1] + b2 * g.epi.batch_stride[2];
+    const int       em0 = m0, en0 = n0; // the finished tile (m0, n0 move on to the next one below)
+    bool            has_next = false;
+    if constexpr (PERSIST)
+    {
+        walk_it++;
+        const int L = walk_it * (int) gridDim.x + walk_first;
+        has_next = L < walk_total;
+        if (has_next)
+        {
+            __syncthreads(); // the slowest wavefront has taken its last fragments out of the ring
+            locate(L % tiles_total, L / tiles_total);
+            setup_ptrs();
+            issue_prologue();
+        }
+    }
+    // (PERSIST: the epilogue's lane- and wavefront-dependent values are derived from laundered copies, so that the
+    // compiler does not hoist them out of the walk over tiles and keep them in registers through the main loop)
+    int elane = lane, ewave = wave;
+    if constexpr (PERSIST)
+    {
+        asm volatile("" : "+v"(elane));
+        asm volatile("" : "+s"(ewave));
+    }
+    const int ewm = ewave >> 2, ewn = ewave & 3;
     const long long ldc = g.epi.ld;
     const bool      has_alpha = g.epi.has_alpha != 0;
     const float     alpha = g.epi.alpha;
@@ -568,10 +632,10 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     const int       esz = (dt == DT_FP32) ? 4 : (dt == DT_BF16 ? 2 : 1);
     const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
                            g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
-    const int       kg = lane >> 5;
-    // element offset of this lane's first value in block (0, 0): row m0 + wm * WR + lane % 32, column n0 + wn * 64 + 16 kg
-    const long long lane_elem = c_off + (long long) (m0 + wm * WR + (lane & 31)) * ldc + n0 + wn * 64 + kg * 16;
-    // block (i, j) -> the lane's 16 values after the power-of-two factors and relu
+    const int       kg = elane >> 5;
+    // element offset of this elane's first value in block (0, 0): row em0 + ewm * WR + elane % 32, column en0 + ewn * 64 + 16 kg
+    const long long lane_elem = c_off + (long long) (em0 + ewm * WR + (elane & 31)) * ldc + en0 + ewn * 64 + kg * 16;
+    // block (i, j) -> the elane's 16 values after the power-of-two factors and relu
     auto gather = [&](int i, int j, float (&val)[16], auto raw_c) __attribute__((always_inline))
     {
 #pragma unroll
@@ -593,7 +657,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         if (col_exp)
         {
 #pragma unroll
-            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[RG ? min(n0 + wn * 64 + j * 32 + kg * 16 + c, g.N - 1) : n0 + wn * 64 + j * 32 + kg * 16 + c]);
+            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[RG ? min(en0 + ewn * 64 + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * 64 + j * 32 + kg * 16 + c]);
         }
         if (relu)
         {
@@ -605,18 +669,19 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     typedef uint32_t e_v4u __attribute__((ext_vector_type(4)));
     typedef float    e_v2f __attribute__((ext_vector_type(2)));
     typedef __bf16   e_v2bf __attribute__((ext_vector_type(2)));
-    // Converted values pass through LDS on their way out (the ring is idle by now): a lane holds 16 columns of one row, and
+    // Converted values pass through LDS on their way out (the ring is idle by now): a elane holds 16 columns of one row, and
     // stored from there a 128-byte line of the output would arrive as four to eight separate pieces.  Each wavefront stages
     // one 32-row block of its 64 columns (16-byte chunks XOR-swizzled by row, conflict-free both ways) and stores it back
     // with consecutive lanes on consecutive chunks of a row: whole lines per request.
     auto walk_to = [&](auto esz_c, auto raw_c, uint8_t* outb, long long pitch, auto pack) __attribute__((always_inline))
     {
-        constexpr int ESZ = decltype(esz_c)::value; // bytes per output element = 16-byte chunks per lane and block
+        constexpr int ESZ = decltype(esz_c)::value; // bytes per output element = 16-byte chunks per elane and block
         constexpr int RB = 64 * ESZ, CPR = RB / 16, NRD = RB / 32;
-        char*         stg = lds + wave * (32 * RB);
-        const int     row = lane & 31, swz = (row * CPR / 16) & (CPR - 1);
+        // (PERSIST: behind the ring, which already holds the next tile; 1- and 2-byte outputs only, the host sees to that)
+        char*         stg = lds + (PERSIST && ESZ <= 2 ? FNST * STAGE : 0) + ewave * (32 * RB);
+        const int     row = elane & 31, swz = (row * CPR / 16) & (CPR - 1);
         constexpr bool RAW = decltype(raw_c)::value; // partial sums of a k-slice: no factors, no relu
-        __syncthreads(); // the slowest wavefront has taken its last fragments out of the ring
+        if constexpr (!PERSIST) __syncthreads(); // the slowest wavefront has taken its last fragments out of the ring
 #pragma unroll
         for (int i = 0; i < NI; i++)
         {
@@ -637,9 +702,9 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #pragma unroll
             for (int r = 0; r < NRD; r++)
             {
-                const int   q = r * 64 + lane, rr = q / CPR, lc = q % CPR;
+                const int   q = r * 64 + elane, rr = q / CPR, lc = q % CPR;
                 const e_v4u v = *(const e_v4u*) (stg + rr * RB + ((lc ^ ((rr * CPR / 16) & (CPR - 1))) << 4));
-                if ((!RAGGED_M || m0 + wm * WR + i * 32 + rr < g.M) && (!RG || n0 + wn * 64 + lc * (16 / ESZ) < g.N))
+                if ((!RAGGED_M || em0 + ewm * WR + i * 32 + rr < g.M) && (!RG || en0 + ewn * 64 + lc * (16 / ESZ) < g.N))
                     __builtin_nontemporal_store(v, (e_v4u*) (outb + (long long) (i * 32 + rr) * pitch + lc * 16));
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -650,18 +715,18 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     auto walk = [&](auto esz_c, auto pack) __attribute__((always_inline))
     {
         constexpr int ESZ = decltype(esz_c)::value;
-        walk_to(esz_c, std::false_type(), (uint8_t*) g.epi.out + (c_off + (long long) (m0 + wm * WR) * ldc + n0 + wn * 64) * ESZ, ldc * ESZ, pack);
+        walk_to(esz_c, std::false_type(), (uint8_t*) g.epi.out + (c_off + (long long) (em0 + ewm * WR) * ldc + en0 + ewn * 64) * ESZ, ldc * ESZ, pack);
     };
-    if (g.split_k > 1)
+    if (!PERSIST && g.split_k > 1)
     {
         // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
-        float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N + (long long) (m0 + wm * WR) * g.N + n0 + wn * 64;
+        float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N + (long long) (em0 + ewm * WR) * g.N + en0 + ewn * 64;
         walk_to(std::integral_constant<int, 4>(), std::true_type(), (uint8_t*) ws, (long long) g.N * 4, [&](const float (&val)[16], uint32_t (&pk)[16]) __attribute__((always_inline)) {
 #pragma unroll
             for (int c = 0; c < 16; c++) pk[c] = __float_as_uint(val[c]);
         });
     }
-    else if (dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
+    else if (!PERSIST && dt == DT_FP32 && !(g.epi.fused && (g.epi.cast.clip_fp || g.epi.cast.ftz)))
         walk(std::integral_constant<int, 4>(), [&](const float (&val)[16], uint32_t (&pk)[16]) __attribute__((always_inline)) {
 #pragma unroll
             for (int c = 0; c < 16; c++) pk[c] = __float_as_uint(val[c]);
@@ -669,7 +734,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     else if (dt == DT_BF16 && g.epi.fast_cast)
         // bf16, round to nearest even: v_cvt_pk_bf16_f32 gives the reference's code for every input except NaN (checked over
         // all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x| over
-        // the lane's 16 values detects them and the block is then converted element by element
+        // the elane's 16 values detects them and the block is then converted element by element
         walk(std::integral_constant<int, 2>(), [&](const float (&val)[16], uint32_t (&pk)[8]) __attribute__((always_inline)) {
             float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -725,7 +790,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         else
             fp8_store(std::integral_constant<int, 2>());
     }
-    else
+    else if (!PERSIST)
     {
         // rare cast settings: element-wise through the out-of-line generic converter (which applies relu itself)
 #pragma unroll 1
@@ -758,12 +823,14 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 {
                     float x = val[c];
                     if (has_alpha) x *= alpha;
-                    if (col_exp) x *= pow2_of(col_exp[RG ? min(n0 + wn * 64 + j * 32 + kg * 16 + c, g.N - 1) : n0 + wn * 64 + j * 32 + kg * 16 + c]);
-                    if ((!RAGGED_M || m0 + wm * WR + i * 32 + (lane & 31) < g.M) && (!RG || n0 + wn * 64 + j * 32 + kg * 16 < g.N)) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
+                    if (col_exp) x *= pow2_of(col_exp[RG ? min(en0 + ewn * 64 + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * 64 + j * 32 + kg * 16 + c]);
+                    if ((!RAGGED_M || em0 + ewm * WR + i * 32 + (elane & 31) < g.M) && (!RG || en0 + ewn * 64 + j * 32 + kg * 16 < g.N)) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
                 }
             }
     }
     (void) esz;
+    if (!PERSIST || !has_next) break;
+    } // walk over tiles
 }
 
 

@@ -469,3 +469,42 @@ def test_fp32_three_part_path_steps_aside_for_inf_and_nan(calc, orc):
     assert inf.any() and np.array_equal(got[inf], want[inf])
     fin = np.isfinite(want)
     assert rel_frobenius(got[fin], want[fin]) <= 1e-4
+
+
+PERSISTENT = [  # op, dtA, bA, dtB, bB, out_dt, out_bias, M, N, K, batch, rows per reference launch
+    (abi.OP_AB, abi.FP8_143, 7, abi.FP8_143, 7, abi.BF16, 0, 4096, 8192, 384, 1, 1024),      # 16 x 32 tiles: 8 x 4 blocks per XCD
+    (abi.OP_ABT, abi.FP8_152, 15, abi.FP8_143, 11, abi.FP8_143, 7, 2560, 13312, 512, 1, 1280),  # 10 x 52 tiles: row-major walk
+    (abi.OP_AB, abi.FP8_143, 7, abi.FP8_152, 15, abi.FP8_152, 15, 1280, 13312, 384, 2, 1280),   # two batch elements, B broadcast
+]
+
+
+@pytest.mark.parametrize("op,dtA,bA,dtB,bB,out_dt,out_bias,M,N,K,batch,rows", PERSISTENT)
+def test_fp8_persistent_walk_equals_tile_by_tile_launches(calc, orc, op, dtA, bA, dtB, bB, out_dt, out_bias, M, N, K, batch, rows):
+    """Problems with at least 512 tiles take the kernel whose workgroups walk over tiles (next tile's first stages requested
+    before the finished tile's epilogue).  The same problem launched slab by slab (fewer than 512 tiles per launch: one
+    workgroup per tile, the kernel the other tests hold against the oracle) must give the same output codes."""
+    import torch
+    rng = np.random.default_rng(77)
+    a = random_operand(rng, dtA, M * K * batch, orc, bA)
+    b = random_operand(rng, dtB, N * K, orc, bB, scale=0.05)
+    col = torch.from_numpy(rng.integers(-3, 4, N).astype(np.int32)).cuda()
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    td = torch.int16 if out_dt == abi.BF16 else torch.uint8
+    bsz = [K, N] if op == abi.OP_ABT else [N, K]
+    W = MmeSimTensor(bsz + ([1] if batch > 1 else []), 3 if batch > 1 else 2, dtB, tb, bB)
+    epi = Epilogue(scale_exp=-4, col_scale_exp=col, clipFp=True)
+
+    whole = torch.zeros(M * N * batch, dtype=td, device="cuda")
+    X = MmeSimTensor([K, M] + ([batch] if batch > 1 else []), 3 if batch > 1 else 2, dtA, ta, bA)
+    calc.doBatchGemm(MmeSimTensor([N, M] + ([batch] if batch > 1 else []), 3 if batch > 1 else 2, out_dt, whole, out_bias), X, W, op, epilogue=epi)
+
+    W2 = MmeSimTensor(bsz, 2, dtB, tb, bB)
+    parts = torch.zeros(M * N * batch, dtype=td, device="cuda")
+    assert (rows // 256) * (N // 256) < 512 and (M * batch) % rows == 0
+    for r0 in range(0, M * batch, rows):
+        Xs = MmeSimTensor([K, rows], 2, dtA, ta[r0 * K:(r0 + rows) * K], bA)
+        calc.doBatchGemm(MmeSimTensor([N, rows], 2, out_dt, parts[r0 * N:(r0 + rows) * N], out_bias), Xs, W2, op, epilogue=epi)
+    calc.synchronize()
+    got, want = whole.cpu().numpy(), parts.cpu().numpy()
+    assert np.count_nonzero(want) > want.size // 2
+    assert np.array_equal(got, want)
