@@ -242,9 +242,9 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
     if (tm == 128) return launch_gemm_large_tile_128(p, grid, s);
     if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return p.dtype == DT_BF16 ? launch_conv_bf16(p, grid, s) : launch_gemm_large_tile_conv_fp8(p, grid, s);
+    if (p.A.k_contig && gemm_large_tile_persistent_applicable(p)) return launch_gemm_large_tile_persistent(p, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     if (!p.A.k_contig) return launch_gemm_large_tile_fp8_at(p, grid, s);
-    if (gemm_large_tile_persistent_applicable(p)) return launch_gemm_large_tile_persistent(p, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {
         case 0: return launch_fmt<0>(p, grid, s);

@@ -1,4 +1,4 @@
-// gemm_large_tile_persistent.hip -- the large-tile fp8 GEMM for problems with several tiles per compute unit: 256
+// gemm_large_tile_persistent.hip -- the large-tile fp8 / bf16 GEMM for problems with several tiles per compute unit: 256
 // workgroups walk over the tiles, and each requests the first stages of its next tile before it converts and stores the
 // finished one, so that pipeline fill and epilogue overlap (gemm_large_tile_impl.hpp, PERSIST).
 // Replaces, for these shapes, doGemmWorkerFloat + Gaudi3Fp8Fma::fma_vec of the reference
@@ -17,6 +17,13 @@ __global__ __launch_bounds__(512) void gemm_fp8_persistent_kernel(GemmProblem g_
 {
     (void) g_by_value;
     gemm_fast_body<1, FMT, B_KC, 0, FBM, false, true>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+}
+
+template<bool B_KC>
+__global__ __launch_bounds__(512) void gemm_bf16_persistent_kernel(GemmProblem g_by_value)
+{
+    (void) g_by_value;
+    gemm_fast_body<2, 0, B_KC, 0, FBM, false, true>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
 }
 
 template<class K>
@@ -41,7 +48,7 @@ hipError_t launch_fmt(const GemmProblem& p, hipStream_t s)
 }
 } // namespace
 
-// whole 256 x 256 tiles of a plain fp8 GEMM with A k-contiguous, at least two rounds of tiles on a 256-CU device, fused
+// whole 256 x 256 tiles of a plain fp8 or bf16 GEMM with A k-contiguous, at least two rounds of tiles on a 256-CU device, fused
 // bf16 / fp8 output through the fast converters, no split-k
 bool gemm_large_tile_persistent_applicable(const GemmProblem& p)
 {
@@ -52,7 +59,7 @@ bool gemm_large_tile_persistent_applicable(const GemmProblem& p)
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = -1;
     }
     if (cus != PERSIST_WGS) return false;
-    if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152) || p.tile_m == 128 || p.split_k > 1) return false;
+    if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152 || p.dtype == DT_BF16) || p.tile_m == 128 || p.split_k > 1) return false;
     if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN || !p.A.k_contig) return false;
     if (p.M % FBM || p.N % FBN) return false;
     if (!p.epi.fused || !p.epi.fast_cast) return false;
@@ -63,6 +70,12 @@ bool gemm_large_tile_persistent_applicable(const GemmProblem& p)
 
 hipError_t launch_gemm_large_tile_persistent(const GemmProblem& p, hipStream_t s)
 {
+    if (p.dtype == DT_BF16)
+    {
+        static bool attr_done[2] = {false, false};
+        return p.B.k_contig ? launch_persistent(gemm_bf16_persistent_kernel<true>, attr_done[0], p, s)
+                            : launch_persistent(gemm_bf16_persistent_kernel<false>, attr_done[1], p, s);
+    }
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {
         case 0: return launch_fmt<0>(p, s);

@@ -475,11 +475,13 @@ PERSISTENT = [  # op, dtA, bA, dtB, bB, out_dt, out_bias, M, N, K, batch, rows p
     (abi.OP_AB, abi.FP8_143, 7, abi.FP8_143, 7, abi.BF16, 0, 4096, 8192, 384, 1, 1024),      # 16 x 32 tiles: 8 x 4 blocks per XCD
     (abi.OP_ABT, abi.FP8_152, 15, abi.FP8_143, 11, abi.FP8_143, 7, 2560, 13312, 512, 1, 1280),  # 10 x 52 tiles: row-major walk
     (abi.OP_AB, abi.FP8_143, 7, abi.FP8_152, 15, abi.FP8_152, 15, 1280, 13312, 384, 2, 1280),   # two batch elements, B broadcast
+    (abi.OP_AB, abi.BF16, 0, abi.BF16, 0, abi.BF16, 0, 4096, 8192, 192, 1, 1024),               # bf16 operands
+    (abi.OP_ABT, abi.BF16, 0, abi.BF16, 0, abi.FP8_143, 7, 2560, 13312, 256, 1, 1280),
 ]
 
 
 @pytest.mark.parametrize("op,dtA,bA,dtB,bB,out_dt,out_bias,M,N,K,batch,rows", PERSISTENT)
-def test_fp8_persistent_walk_equals_tile_by_tile_launches(calc, orc, op, dtA, bA, dtB, bB, out_dt, out_bias, M, N, K, batch, rows):
+def test_persistent_walk_equals_tile_by_tile_launches(calc, orc, op, dtA, bA, dtB, bB, out_dt, out_bias, M, N, K, batch, rows):
     """Problems with at least 512 tiles take the kernel whose workgroups walk over tiles (next tile's first stages requested
     before the finished tile's epilogue).  The same problem launched slab by slab (fewer than 512 tiles per launch: one
     workgroup per tile, the kernel the other tests hold against the oracle) must give the same output codes."""
@@ -488,7 +490,8 @@ def test_fp8_persistent_walk_equals_tile_by_tile_launches(calc, orc, op, dtA, bA
     a = random_operand(rng, dtA, M * K * batch, orc, bA)
     b = random_operand(rng, dtB, N * K, orc, bB, scale=0.05)
     col = torch.from_numpy(rng.integers(-3, 4, N).astype(np.int32)).cuda()
-    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    ta = torch.from_numpy(a.view(np.int16) if dtA == abi.BF16 else a).cuda()
+    tb = torch.from_numpy(b.view(np.int16) if dtB == abi.BF16 else b).cuda()
     td = torch.int16 if out_dt == abi.BF16 else torch.uint8
     bsz = [K, N] if op == abi.OP_ABT else [N, K]
     W = MmeSimTensor(bsz + ([1] if batch > 1 else []), 3 if batch > 1 else 2, dtB, tb, bB)
