@@ -23,6 +23,7 @@
 
 #include <array>
 #include <cstdint>
+#include <cstring>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -98,6 +99,45 @@ struct ConvolutionParams
     }
 };
 
+/* stand-alone 2-d matrix with the accessors of the reference's Matrix (mme/mme_reference/mme_reference.h:60-104) that
+ * doGemm reads: getElementType(), data(), getMatrix().getHeight() / getWidth().  Row-major height x width; owns a zeroed
+ * buffer when no data pointer is given, otherwise copies or wraps the caller's (shouldCopyData), like the reference's
+ * first constructor (mme_reference_impl.cpp:17-26). */
+class Matrix
+{
+public:
+    struct Shape
+    {
+        uint64_t height = 0, width = 0;
+        uint64_t getHeight() const { return height; }
+        uint64_t getWidth() const { return width; }
+    };
+    Matrix(int type, uint64_t height, uint64_t width, void* data_ = nullptr, bool shouldCopyData = true) : m_type(type)
+    {
+        m_shape.height = height;
+        m_shape.width = width;
+        const size_t es = (type == MME_HIP_FP8_143 || type == MME_HIP_FP8_152) ? 1 : ((type == MME_HIP_BF16 || type == MME_HIP_FP16 || type == MME_HIP_UFP16) ? 2 : 4);
+        const size_t bytes = (size_t) (height * width) * es;
+        if (data_ && !shouldCopyData) m_data = (unsigned char*) data_;
+        else
+        {
+            m_owned.reset(new unsigned char[bytes ? bytes : 1]());
+            if (data_ && bytes) std::memcpy(m_owned.get(), data_, bytes);
+            m_data = m_owned.get();
+        }
+    }
+    const Shape&         getMatrix() const { return m_shape; }
+    int                  getElementType() const { return m_type; }
+    unsigned char*       data() { return m_data; }
+    const unsigned char* data() const { return m_data; }
+
+private:
+    int                              m_type;
+    Shape                            m_shape;
+    unsigned char*                   m_data = nullptr;
+    std::unique_ptr<unsigned char[]> m_owned;
+};
+
 /* fused descale + relu + cast behind a device-resident contraction (mme_hip_epilogue) */
 typedef mme_hip_epilogue Epilogue;
 
@@ -117,6 +157,36 @@ public:
 
     /* mme_reference.h:122 */
     void limitNumOfThreads(unsigned numOfThreads) { check(mme_hip_limit_num_of_threads(m_h, numOfThreads)); }
+
+    /* mme_reference.h:126-138, mme_reference_impl.cpp:541-596: output (M x N) = op(A) * op(B) on row-major matrices;
+     * transposeA / transposeB say that the matrix handed in is the transpose of the factor.  The exponent biases and
+     * inf/NaN modes of the operands are arguments here (a Matrix carries none).  M is the reference's Matrix or
+     * MmeHip::Matrix: read through getElementType(), data(), getMatrix().getHeight() / getWidth(). */
+    template<class M>
+    void doGemm(M& output, const M& inputA, const M& inputB, bool transposeA, bool transposeB, int rm = MME_HIP_RM_NEAREST_EVEN,
+                unsigned fpBiasA = 0, unsigned fpBiasB = 0, bool clipFp = false, bool clipFpInfIn = false,
+                int infNanModeA = MME_HIP_FULL_INF_NAN, int infNanModeB = MME_HIP_FULL_INF_NAN, int* zeroPoints = nullptr)
+    {
+        no_zero_points(zeroPoints);
+        const mme_hip_tensor o = pod_matrix(output, 0, MME_HIP_FULL_INF_NAN), a = pod_matrix(inputA, fpBiasA, infNanModeA),
+                             b = pod_matrix(inputB, fpBiasB, infNanModeB);
+        const int op = transposeA ? (transposeB ? MME_HIP_OP_ATBT : MME_HIP_OP_ATB) : (transposeB ? MME_HIP_OP_ABT : MME_HIP_OP_AB);
+        check(mme_hip_batch_gemm(m_h, &o, &a, &b, op, rm, clipFp, clipFpInfIn));
+    }
+
+    /* mme_reference.h:140 (memcpy / transpose through the MME's DMA mode) and :180-187 (the integer path's requantisation):
+     * not part of this library; they throw like any other unsupported request, so that a CPUCalculator built on this class
+     * links without the reference's CPU implementation. */
+    template<class T>
+    void doDma(T&, const T&, int)
+    {
+        throw MMEStackException("doDma is not built in this library (memcpy / transpose are not contractions)", MME_HIP_EUNSUPPORTED);
+    }
+    template<class PT>
+    void activationGemmlowp(PT, PT, PT, PT, bool, int, const void*)
+    {
+        throw MMEStackException("activationGemmlowp belongs to the integer path, which is not built in this library", MME_HIP_EUNSUPPORTED);
+    }
 
     /* mme_reference.h:142-149.  zeroPoints belongs to the integer path and must be null. */
     template<class T>
@@ -210,6 +280,28 @@ private:
         d.dtype = (int32_t) t.getElementType();
         d.fp_bias = t.getFpBias();
         d.inf_nan_mode = (int32_t) t.getInfNanMode();
+        return d;
+    }
+    template<class M>
+    static mme_hip_tensor pod_matrix(const M& m, unsigned fpBias, int infNanMode)
+    {
+        mme_hip_tensor d;
+        const uint64_t h = m.getMatrix().getHeight(), w = m.getMatrix().getWidth();
+        if (h >= (1ull << 31) || w >= (1ull << 31) || h * w >= (1ull << 31)) throw MMEStackException("matrix: more than 2^31 elements", MME_HIP_EINVAL);
+        d.data = (void*) m.data();
+        for (int i = 0; i < MME_HIP_MAX_TENSOR_DIMS; i++)
+        {
+            d.sizes[i] = 1;
+            d.strides[i] = (uint32_t) (h * w);
+        }
+        d.sizes[0] = (uint32_t) w;
+        d.sizes[1] = (uint32_t) h;
+        d.strides[0] = 1;
+        d.strides[1] = (uint32_t) w;
+        d.dim = 2;
+        d.dtype = (int32_t) m.getElementType();
+        d.fp_bias = fpBias;
+        d.inf_nan_mode = infNanMode;
         return d;
     }
     template<class P>

@@ -1,5 +1,5 @@
 // Known-answer tests of the C++ surface (include/mme_hip_calculator.h) written the way the reference's own unit tests
-// drive CPUCalculator (mme/tests/unit_tests/mme_unit_test.cpp:67-172, 394-519): same shapes, values and expectations,
+// drive CPUCalculator (mme/tests/unit_tests/mme_unit_test.cpp:67-172, 394-519, 539-575): same shapes, values and expectations,
 // host tensors, synchronous calls.  Needs a GPU.  Prints one line per case and exits non-zero on the first failure.
 #include "mme_hip_calculator.h"
 
@@ -207,6 +207,82 @@ static void memory_write_reductions(Calculator& calculator)
     EXPECT(m16[0] == o16[0] && m16[1] == o16[1]);
 }
 
+// mme_unit_test.cpp:84-106: the Matrix form of the 5-term product, 1 x 5 times 5 x 1
+static void reference_gemm_api_simple_test_fp32(Calculator& calculator)
+{
+    std::vector<float> data(5, 10.0f);
+    MmeHip::Matrix     a(MME_HIP_FP32, 1, 5, data.data()), b(MME_HIP_FP32, 5, 1, data.data()), y(MME_HIP_FP32, 1, 1);
+    calculator.doGemm(y, a, b, false, false);
+    float got;
+    std::memcpy(&got, y.data(), 4);
+    EXPECT(got == 500.0f);
+}
+
+// mme_unit_test.cpp:539-575: fp16 operands, A handed in transposed (128 x 128), B 128 x 256, every element 10.  The
+// reference's test asserts nothing; the values follow from the arithmetic: 128 products of 10 * 10 with the IEEE exponent
+// bias, and with the call's default bias 0 every operand is 10 * 2^15.  All four transpose flags on a matrix with
+// distinct entries: y = op(A) op(B) against a host loop.
+static void reference_gemm_api(Calculator& calculator)
+{
+    const unsigned        M = 128, K = 128, N = 256;
+    std::vector<uint16_t> da(K * M, 0x4900), db(K * N, 0x4900); // fp16 10.0
+    MmeHip::Matrix        a(MME_HIP_FP16, K, M, da.data()), b(MME_HIP_FP16, K, N, db.data()), y(MME_HIP_FP32, M, N);
+    calculator.doGemm(y, a, b, true, false, MME_HIP_RM_NEAREST_EVEN, 15, 15);
+    const float* out = (const float*) y.data();
+    bool         all = true;
+    for (unsigned i = 0; i < M * N; i++) all = all && out[i] == 12800.0f;
+    EXPECT(all);
+    calculator.doGemm(y, a, b, true, false);
+    all = true;
+    for (unsigned i = 0; i < M * N; i++) all = all && out[i] == 12800.0f * 1073741824.0f;
+    EXPECT(all);
+    // small integers: exact in bf16 and in every accumulation order
+    const unsigned     m = 3, k = 4, n = 2;
+    std::vector<float> A(m * k), B(k * n), want(m * n, 0.0f);
+    for (unsigned i = 0; i < m * k; i++) A[i] = (float) (i % 7) - 3.0f;
+    for (unsigned i = 0; i < k * n; i++) B[i] = (float) (i % 5) - 2.0f;
+    for (unsigned i = 0; i < m; i++)
+        for (unsigned j = 0; j < n; j++)
+            for (unsigned l = 0; l < k; l++) want[i * n + j] += A[i * k + l] * B[l * n + j];
+    for (int ta = 0; ta < 2; ta++)
+        for (int tb = 0; tb < 2; tb++)
+        {
+            std::vector<uint16_t> ha(m * k), hb(k * n);
+            for (unsigned i = 0; i < m; i++)
+                for (unsigned l = 0; l < k; l++) ha[ta ? l * m + i : i * k + l] = bf16_of(A[i * k + l]);
+            for (unsigned l = 0; l < k; l++)
+                for (unsigned j = 0; j < n; j++) hb[tb ? j * k + l : l * n + j] = bf16_of(B[l * n + j]);
+            MmeHip::Matrix ma(MME_HIP_BF16, ta ? k : m, ta ? m : k, ha.data(), false), mb(MME_HIP_BF16, tb ? n : k, tb ? k : n, hb.data(), false),
+                my(MME_HIP_FP32, m, n);
+            calculator.doGemm(my, ma, mb, ta != 0, tb != 0);
+            EXPECT(std::memcmp(my.data(), want.data(), m * n * 4) == 0);
+        }
+    // the methods outside the path throw instead of computing
+    bool thrown = false;
+    try
+    {
+        float  v = 0.0f;
+        Tensor t({1, 1, 1, 1, 1}, 2, MME_HIP_FP32, &v);
+        calculator.doDma(t, t, MME_HIP_OP_AB);
+    }
+    catch (const MMEStackException& e)
+    {
+        thrown = e.status == MME_HIP_EUNSUPPORTED;
+    }
+    EXPECT(thrown);
+    thrown = false;
+    try
+    {
+        std::shared_ptr<Tensor> none;
+        calculator.activationGemmlowp(none, none, none, none, false, MME_HIP_RM_NEAREST_EVEN, nullptr);
+    }
+    catch (const MMEStackException& e)
+    {
+        thrown = e.status == MME_HIP_EUNSUPPORTED;
+    }
+    EXPECT(thrown);
+}
+
 // error conventions: what MME_ASSERT rejects must throw (mme_reference_impl.cpp:465-467, 591)
 static void error_conventions(Calculator& calculator)
 {
@@ -264,6 +340,8 @@ int main()
                      {"fp16_convert_and_gemm", fp16_convert_and_gemm},
                      {"tf32_operand_clip", tf32_operand_clip},
                      {"memory_write_reductions", memory_write_reductions},
+                     {"reference_gemm_api_simple_test_fp32", reference_gemm_api_simple_test_fp32},
+                     {"reference_gemm_api", reference_gemm_api},
                      {"error_conventions", error_conventions}};
         for (auto& c : cases)
         {

@@ -68,3 +68,22 @@ def test_headers_compile_as_c_and_cpp(tmp_path):
                        'void f(MmeHip::Calculator& c, MmeHip::Tensor& o, const MmeHip::Tensor& a, const MmeHip::Tensor& b, const MmeHip::ConvolutionParams& p)\n'
                        '{ c.doBatchGemm(o, a, b, MME_HIP_OP_AB); c.doConvolution(o, a, b, o, p, MME_HIP_OP_FWD); c.doBatchGemmDev(o, a, b, MME_HIP_OP_ABT); }\n')
     subprocess.check_call(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-I" + inc, str(cpp_src)])
+
+
+def test_reference_side_stub_compiles_against_the_reference_headers():
+    """include/reference_stub/mme_reference_hip.cpp defines every CPUCalculator method of mme/mme_reference/mme_reference.h:108-191
+    on top of MmeHip::Calculator; with the reference tree present it must pass the compiler's front end against the
+    reference's own headers (MmeSimTensor, Matrix, ConvolutionParams, the enums)."""
+    import subprocess
+    ref = os.environ.get("MME_REFERENCE_ROOT", "/root/reference")
+    if not os.path.isdir(os.path.join(ref, "mme", "mme_reference")):
+        pytest.skip("the reference tree is not present")
+    inc = ["mme", "mme/include", "mme/mme_reference", "mme/src/mme_common", "mme/src", "3rd-parties", "3rd-parties/spdlog/include",
+           "coral-sim/header/gaudi3/fs_core", "coral-sim/header/gaudi2/fs_core"]
+    cmd = ["g++", "-std=c++17", "-fsyntax-only", "-w", "-I" + os.path.join(ROOT, "include")] + ["-I" + os.path.join(ref, i) for i in inc]
+    subprocess.check_call(cmd + [os.path.join(ROOT, "include", "reference_stub", "mme_reference_hip.cpp")])
+    # every public method of the class is defined by the stub
+    text = open(os.path.join(ROOT, "include", "reference_stub", "mme_reference_hip.cpp")).read()
+    for m in ("CPUCalculator::CPUCalculator", "CPUCalculator::~CPUCalculator", "limitNumOfThreads", "doGemm", "doDma", "doBatchGemm", "doConvolution",
+              "doActivation", "doMemoryWrite", "activationGemmlowp"):
+        assert m in text

@@ -176,10 +176,8 @@ GATHER_CASES = [
 @pytest.mark.parametrize("op", [abi.OP_FWD, abi.OP_DEDX])
 @pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP16, 15), (abi.FP16, 11), (abi.FP8_143, 7), (abi.FP8_143, 11), (abi.FP8_152, 15)])
 def test_conv_large_tile_gather_vs_oracle(calc, orc, case, op, dt, bias):
-    if op == abi.OP_DEDX and case[0] < 128:
-        pytest.skip("dedx has C output columns: the large-tile kernel takes 128 or more")
-    if case[6] == 1 and op == abi.OP_FWD:
-        pass  # K * taps = 256 channels: 8 stages
+    # (dedx has C output columns and the large-tile kernel takes 128 or more: the dedx of the 64-channel case runs on the
+    # general kernel, and is held to the same bounds)
     got, want = _run(calc, orc, case, dt, bias, op, device=True)
     assert rel_frobenius(got, want) <= TOL[dt]
     assert rel_frobenius(got, want) <= 1e-4

@@ -17,4 +17,4 @@ def test_cpp_known_answers():
     text = r.stdout.decode(errors="replace")
     print(text)
     assert r.returncode == 0, text
-    assert text.count("ok    ") == 10 and "FAILED" not in text
+    assert text.count("ok    ") == 12 and "FAILED" not in text
