@@ -13,17 +13,36 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-tar
          "-Wno-unused-command-line-argument", "-Wno-unknown-attributes"]
 
 
-def build_library(verbose=False, jobs=8):
-    """Compile every HIP source and link the shared library.  Always recompiles."""
+def _includes(path, seen=None):
+    """The files a source includes from this directory, transitively (for the only_changed mode)."""
+    import re
+    seen = set() if seen is None else seen
+    with open(path) as f:
+        names = re.findall(r'#include\s+"([^"]+)"', f.read())
+    for name in names:
+        dep = os.path.normpath(os.path.join(os.path.dirname(path), name))
+        if os.path.exists(dep) and dep not in seen:
+            seen.add(dep)
+            _includes(dep, seen)
+    return seen
+
+
+def build_library(verbose=False, jobs=8, only_changed=False):
+    """Compile every HIP source and link the shared library.  Recompiles everything unless only_changed is set (then a
+    source is skipped when its object is newer than the source and every header it includes)."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objs, procs = [], []
     for src in SOURCES:
         obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        objs.append(obj)
+        if only_changed and os.path.exists(obj):
+            deps = [os.path.join(CSRC, src)] + sorted(_includes(os.path.join(CSRC, src)))
+            if all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps):
+                continue
         cmd = [hipcc] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
-        objs.append(obj)
         if len(procs) >= jobs:
             _wait(procs)
     _wait(procs)
@@ -59,5 +78,5 @@ def _wait(procs):
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_library(verbose=True, only_changed="--changed" in sys.argv))
     print(build_cpp_tests())

@@ -225,15 +225,21 @@ class HipCalculator:
         self._check(self._lib.mme_hip_set_stream(self._h, hip_stream))
         self._caller_stream = bool(hip_stream)
 
-    def _after_torch(self):
+    def _after_torch(self, *device_tensors):
         # the calculator's own stream does not synchronise with any other: make it wait (on the device) for the fills and
-        # copies that produced the operands on torch's current stream
+        # copies that produced the operands on torch's current stream, and tell torch's allocator that the operands are in
+        # use on that stream, so that a temporary passed inline is not handed to the next allocation while a kernel still
+        # reads it.  Results may be consumed on torch's stream after synchronize().
         if self._caller_stream:
             return
         import torch
+        own = torch.cuda.ExternalStream(self.stream())
         ev = torch.cuda.Event()
         ev.record()
-        torch.cuda.ExternalStream(self.stream()).wait_event(ev)
+        own.wait_event(ev)
+        for t in device_tensors:
+            if t is not None and getattr(t, "is_cuda", False):
+                t.record_stream(own)
 
     def setFp8SpecialsPolicy(self, policy):
         self._check(self._lib.mme_hip_set_fp8_specials_policy(self._h, policy))
@@ -241,7 +247,7 @@ class HipCalculator:
     def castFromFp32(self, out, out_dtype, src, n, fpBias=0, infNanMode=FULL_INF_NAN, scale_exp=0, col_scale_exp=None,
                      n_cols=0, relu=False, rm=RM_NEAREST_EVEN, clipFp=False, clipInfIn=False, flushDenorms=False):
         """Flat quantise / cast on device buffers (torch tensors)."""
-        self._after_torch()
+        self._after_torch(out, src, col_scale_exp)
         self._check(self._lib.mme_hip_cast_from_fp32_dev(
             self._h, out.data_ptr(), out_dtype, fpBias, infNanMode, src.data_ptr(), n, scale_exp,
             col_scale_exp.data_ptr() if col_scale_exp is not None else None, n_cols, int(relu), rm, int(clipFp), int(clipInfIn),
@@ -249,13 +255,13 @@ class HipCalculator:
 
     def castToFp32(self, out, src, in_dtype, n, fpBias=0, infNanMode=FULL_INF_NAN, scale_exp=0, col_scale_exp=None, n_cols=0):
         """Flat dequantise on device buffers (torch tensors)."""
-        self._after_torch()
+        self._after_torch(out, src, col_scale_exp)
         self._check(self._lib.mme_hip_cast_to_fp32_dev(
             self._h, out.data_ptr(), src.data_ptr(), in_dtype, fpBias, infNanMode, n, scale_exp,
             col_scale_exp.data_ptr() if col_scale_exp is not None else None, n_cols))
 
     def absmax(self, out, src, n):
-        self._after_torch()
+        self._after_torch(out, src)
         self._check(self._lib.mme_hip_absmax_dev(self._h, out.data_ptr(), src.data_ptr(), n))
 
     def _placement(self, *tensors):
@@ -263,5 +269,5 @@ class HipCalculator:
         if any(dev) and not all(dev):
             raise MMEStackException("tensors of one call must all be host or all be device resident", abi.EINVAL)
         if all(dev):
-            self._after_torch()
+            self._after_torch(*[t.data() for t in tensors])
         return all(dev)

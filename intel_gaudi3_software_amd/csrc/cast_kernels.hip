@@ -651,8 +651,9 @@ hipError_t launch_round_to_tf32(void* out, const void* in, size_t n, int clip, i
 // exact in fp32: the contraction becomes one bf16 contraction over 4 K, operand A laid out as [hi | hi | lo | lo] along k and
 // operand B as [hi | lo | hi | lo].  The copies are dense: (batch, f, 4 K) when the source is k-contiguous, (batch, 4 K, f)
 // otherwise; batch dimensions the source broadcasts (stride 0) have extent 1 in the copy.  A value that is not finite
-// cannot be split (inf * 0 appears among the partial products): it stores `epoch` into *flag and the caller's predicated
-// launches take the fp32 path instead.  V elements per lane along the contiguous index (8 with 16-byte accesses, or 1).
+// cannot be split (inf * 0 appears among the partial products), nor can a value so small that its low part would fall
+// under bf16's normal range (below 2^-100 for fp32, 2^-112 for the 11-bit types): either stores `epoch` into *flag and the
+// caller's predicated launches take the fp32 path instead.  V elements per lane along the contiguous index (8 with 16-byte accesses, or 1).
 // fp32 operands (24 significant bits) take three parts, value = hi + mid + lo of 8 bits each, and six K-blocks: A as
 // [hi | hi | mid | hi | lo | mid], B as [hi | mid | hi | lo | hi | mid]; the three products left out (mid lo, lo mid, lo lo)
 // are below 2^-23 of hi hi, the rounding step of the fp32 accumulation itself.
@@ -704,6 +705,11 @@ __global__ __launch_bounds__(CAST_THREADS) void split_bf16_kernel(uint16_t* __re
             else
                 u = f2u(decode1<DT>(raw[j], a.bias, a.mode));
             special = special || ((u & 0x7F800000u) == 0x7F800000u);
+            // the lowest part ends at the value's last significant bit, 2^-23 (fp32) or 2^-10 (the 11-bit types) below its
+            // exponent, and has to be a normal bf16 number itself (smallest 2^-126) so that no matrix instruction may flush
+            // it: a non-zero value below 2^-100 (fp32) / 2^-112 cannot be split either
+            constexpr uint32_t MIN_EXP_FIELD = DT == DT_FP32 ? 127 - 100 : 127 - 112;
+            special = special || ((u & 0x7FFFFFFFu) != 0 && ((u >> 23) & 0xFFu) < MIN_EXP_FIELD);
             const uint32_t h = u & 0xFFFF0000u;
             hi[j] = h >> 16;
             const float rest = u2f(u) - u2f(h);

@@ -180,6 +180,26 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s)
     const long long nb = (long long) p.batch[0] * p.batch[1] * p.batch[2];
     if (p.M <= 0 || p.N <= 0 || nb <= 0) return hipSuccess;
     hipError_t e;
+    if (nb > 65535)
+    {
+        // the batch index is the grid's y dimension (at most 65535): slice the slowest batch dimension that has an extent,
+        // one launch per slice with the operands' and the output's base pointers moved on
+        const int       d = p.batch[2] > 1 ? 2 : (p.batch[1] > 1 ? 1 : 0);
+        const long long inner = nb / p.batch[d];
+        const int       step = inner >= 65535 ? 1 : (int) (65535 / inner);
+        const int       es = dt_bytes(p.dtype), out_es = p.epi.fused ? dt_bytes(p.epi.out_dtype) : 4;
+        for (int b = 0; b < p.batch[d]; b += step)
+        {
+            GemmProblem q = p;
+            q.batch[d] = p.batch[d] - b < step ? p.batch[d] - b : step;
+            q.A.base = p.A.base + (long long) b * p.A.batch_stride[d] * es;
+            q.B.base = p.B.base + (long long) b * p.B.batch_stride[d] * es;
+            q.epi.out = (char*) p.epi.out + (long long) b * p.epi.batch_stride[d] * out_es;
+            e = launch_gemm(q, s);
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
     if (gemm_large_tile_applicable(p)) e = launch_gemm_large_tile(p, s);
     else
     {

@@ -1156,7 +1156,9 @@ int mme_hip_memory_write(mme_hip_handle h, const mme_hip_tensor* memory, const m
     if (int rc = stage_in(h, sm, memory, true)) return rc;
     if (int rc = stage_in(h, so, &o, true)) return rc;
     if (int rc = mme_hip_memory_write_dev(h, &sm.t, &so.t, reduction_op, reduction_rm, clip_fp)) return rc;
-    return stage_out(h, sm);
+    if (int rc = stage_out(h, sm)) return rc;
+    HIP_TRY(h, hipStreamSynchronize(h->stream));
+    return MME_HIP_OK;
 }
 
 } // extern "C"

@@ -117,6 +117,10 @@ def ref():
         L.ref_compare_elements.argtypes = [vp, vp, vp, C.c_size_t, C.c_int, C.c_uint, C.c_int, C.c_uint]
         L.ref_compare_elements.restype = None
         L.ref_compare_tensors.argtypes = [vp, vp, C.c_uint, C.c_int, vp]
+        if hasattr(L, "ref_compare_elements_partials"):
+            L.ref_compare_elements_partials.argtypes = [vp, vp, vp, C.c_size_t, C.c_uint, C.c_int, C.c_uint, C.c_int, C.c_uint]
+            L.ref_compare_elements_partials.restype = None
+            L.ref_compare_tensors_partials.argtypes = [vp, vp, C.c_uint, C.c_uint, vp]
         L.ref_fma_vec_clip.restype = C.c_uint32
         L.ref_fma_vec_clip.argtypes = [vp, vp, C.c_uint, C.c_int, C.c_int, C.c_uint, C.c_uint] + [C.c_int] * 4
         L.ref_batch_gemm_clip.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int]

@@ -79,6 +79,67 @@ def test_whole_tensors_first_mismatch_and_stride_holes(ref, capsys):
             assert cmp.getDiffElement() == [int(v) for v in diff], raw_index
 
 
+@pytest.mark.parametrize("dt,bias,mode", [(abi.BF16, 0, 0), (abi.FP16, 15, 0), (abi.FP16, 9, 1), (abi.UFP16, 31, 0), (abi.FP32, 0, 0)])
+@pytest.mark.parametrize("num_partials", [2, 3, 5])
+def test_partial_sum_rule_matches_the_reference_class(ref, dt, bias, mode, num_partials):
+    """numPartials > 1: the first tensor holds partial results, the second their sum (tensor_comparator_impl.cpp:373-413).
+    Groups whose rounded fp32 sum equals, nearly equals or misses the second tensor's element, incl. sums that overflow
+    the type, cancel to zero or involve inf / NaN, element by element against the reference's class; then whole tensors."""
+    rng = np.random.default_rng(dt * 10 + num_partials)
+    n = 4000
+    t = NP[abi.DTYPE_SIZE[dt]]
+    bits = 8 * abi.DTYPE_SIZE[dt]
+    from intel_gaudi3_software_amd.comparator import encode_rne
+    default_bias = {abi.FP16: 15, abi.UFP16: 31}.get(dt, 0)
+    vals = (rng.standard_normal((n, num_partials)) * np.exp2(rng.integers(-6, 7, (n, 1)))).astype(np.float32)
+    if dt == abi.UFP16:
+        vals = np.abs(vals)
+    vals[: n // 8] *= np.float32(2.0 ** 14)                      # sums near and beyond fp16's largest value
+    vals[n // 8: n // 4, 1] = -vals[n // 8: n // 4, 0]            # cancellation
+    a = encode_rne(vals.ravel(), dt, default_bias).astype(t)
+    a[rng.integers(0, a.size, 40)] = rng.integers(0, 1 << bits, 40, dtype=np.uint64).astype(t)   # arbitrary codes, inf and NaN among them
+    total = np.zeros(n, np.float32)
+    dec = decode(a, dt, default_bias, 0).reshape(n, num_partials)
+    with np.errstate(invalid="ignore", over="ignore"):
+        for p in range(num_partials):
+            total = (total + dec[:, p]).astype(np.float32)
+    b = encode_rne(total, dt, default_bias).astype(np.int64)
+    b += rng.choice([0, 0, 1, -1, 3, -6, 40, 3000], n)            # equal, a few codes apart, far apart
+    b = (b % (1 << bits)).astype(t)
+    for cd in (1, 27000, 1 << 20):
+        want = np.zeros(n, np.uint8)
+        ref.ref_compare_elements_partials(want.ctypes.data, a.ctypes.data, b.ctypes.data, n, num_partials, dt, bias, mode, cd)
+        cmp = TensorComparator(cd, dt, bias, mode)
+        got = cmp.compare_codes(cmp._sum_partials(np.ascontiguousarray(a.reshape(n, num_partials).T).ravel(), n, num_partials), b)
+        bad = np.flatnonzero(got != want.astype(bool))
+        assert bad.size == 0, (cd, [hex(int(v)) for v in a.reshape(n, num_partials)[bad[0]]], hex(int(b[bad[0]])), bool(want[bad[0]]))
+        assert want.sum() > 0 and (cd > 1 or want.sum() < n)
+    # whole tensors: partials stacked along the last dimension, first mismatch reported by its coordinates in the sum tensor
+    sizes = [6, 5, 4, 1, 1]
+    nb = 120
+    pa = encode_rne((rng.standard_normal(nb * num_partials) * 8).astype(np.float32), dt, default_bias).astype(t)
+    if dt == abi.UFP16:
+        pa = encode_rne(np.abs(rng.standard_normal(nb * num_partials) * 8).astype(np.float32), dt, default_bias).astype(t)
+    cmp = TensorComparator(64, dt, bias, mode)
+    sb = cmp._sum_partials(pa, nb, num_partials).astype(t)
+    ta = MmeSimTensor([6, 5, 4 * num_partials, 1, 1], 3, dt, pa, bias, mode)
+    tb = MmeSimTensor(sizes, 3, dt, sb, bias, mode)
+    diff = np.zeros(5, np.uint32)
+    assert cmp.doCompare(ta, "partials", tb, "sum", numPartials=num_partials)
+    assert ref.ref_compare_tensors_partials(A(ta.desc), A(tb.desc), 64, num_partials, diff.ctypes.data) == 1
+    sb[2 + 6 * 3 + 30 * 1] ^= t(1 << (bits - 2))   # element (2, 3, 1): the exponent's top bit
+    assert not cmp.doCompare(ta, "partials", tb, "sum", numPartials=num_partials, failOnMismatch=False)
+    assert ref.ref_compare_tensors_partials(A(ta.desc), A(tb.desc), 64, num_partials, diff.ctypes.data) == 0
+    assert cmp.getDiffElement() == [int(v) for v in diff] == [2, 3, 1, 0, 0]
+
+
+def test_partial_sums_of_fp8_tensors_are_refused():
+    t8 = MmeSimTensor([4, 1, 1, 1, 1], 1, abi.FP8_143, np.zeros(4, np.uint8), 7)
+    t2 = MmeSimTensor([2, 1, 1, 1, 1], 1, abi.FP8_143, np.zeros(2, np.uint8), 7)
+    with pytest.raises(ValueError):
+        TensorComparator(8, abi.FP8_143, 7).doCompare(t8, "a", t2, "b", numPartials=2)
+
+
 def test_known_cases():
     """Cases that follow from the rule's text: NaN never compares equal, equal infinities do, an infinity against a number
     does not, small values compare by absolute tolerance, large ones by code distance."""

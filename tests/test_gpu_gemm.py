@@ -73,6 +73,17 @@ def test_gemm_aligned_vector_path(calc, orc, op, dtA, dtB, bA, bB, mA, mB):
     assert rel_frobenius(got, want) <= TOL[dtA]
 
 
+@pytest.mark.parametrize("batch,bcast_b", [((70000, 1, 1), True), ((300, 250, 1), False), ((3, 2, 33000), True)])
+def test_gemm_more_than_65535_batch_entries(calc, orc, batch, bcast_b):
+    """More batch entries than one launch's grid holds along its batch axis: the call slices the slowest batch dimension
+    over several launches; every entry against the oracle."""
+    got, want = _run_both(calc, orc, abi.OP_AB, 3, 5, 8, abi.BF16, abi.BF16, 0, 0, 0, 0, batch=batch, bcast_b=bcast_b, seed=31, device=True)
+    assert rel_frobenius(got, want) <= 1e-4
+    per = 15
+    blocks = np.abs(got.reshape(-1, per) - want.reshape(-1, per)).max(axis=1)
+    assert np.all(blocks <= 1e-3 * max(1.0, np.abs(want).max())), int(np.argmax(blocks))
+
+
 def test_gemm_strided_rows_keep_gaps(calc, orc):
     """Row pitches larger than the row (sub-views): gaps in the output keep their previous contents."""
     got, want = _run_both(calc, orc, abi.OP_AB, 9, 10, 20, abi.BF16, abi.BF16, 0, 0, 0, 0, pad=(5, 3, 2), seed=4)
@@ -469,6 +480,43 @@ def test_fp32_three_part_path_steps_aside_for_inf_and_nan(calc, orc):
     assert inf.any() and np.array_equal(got[inf], want[inf])
     fin = np.isfinite(want)
     assert rel_frobenius(got[fin], want[fin]) <= 1e-4
+
+
+@pytest.mark.parametrize("scale_exp", [-115, -126])
+def test_fp32_three_part_path_steps_aside_for_tiny_magnitudes(calc, orc, scale_exp):
+    """fp32 operands below 2^-100: the low bf16 parts of such values would fall under bf16's range (a = 2^-126 (1 + 2^-8)
+    split into bf16 parts loses the 2^-8 entirely), so the contraction must run on the fp32 instantiation.  One operand is
+    scaled by 2^scale_exp, the other by 2^100, so that the products are ordinary numbers: against float64, and bit for bit
+    on one-hot operands with full 24-bit significands."""
+    import torch
+    M, N, K = 256, 256, 1024
+    rng = np.random.default_rng(21)
+    # (random values stay normal fp32 numbers: 2^-115 times a draw; the one-hot values below go down to 2^-126 exactly)
+    a = (rng.standard_normal((M, K)).astype(np.float32) * np.float32(2.0 ** max(scale_exp, -115))).astype(np.float32)
+    b = (rng.standard_normal((K, N)).astype(np.float32) * np.float32(2.0 ** 100)).astype(np.float32)
+    out = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+
+    def run(am, bm):
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, out), MmeSimTensor([K, M], 2, abi.FP32, torch.from_numpy(np.ascontiguousarray(am).ravel()).cuda()),
+                         MmeSimTensor([N, K], 2, abi.FP32, torch.from_numpy(np.ascontiguousarray(bm).ravel()).cuda()), abi.OP_AB)
+        calc.synchronize()
+        return out.cpu().numpy().reshape(M, N).astype(np.float64)
+
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    assert rel_frobenius(run(a, b).ravel(), exact.ravel()) <= 2e-6
+    # one-hot: a holds one value per row position k with all 24 significant bits (the advisor's example has 9), b a power of two
+    a1 = np.zeros((M, K), np.float32)
+    b1 = np.zeros((K, N), np.float32)
+    vals = ((1.0 + rng.integers(1, 1 << 23, K) * 2.0 ** -23) * 2.0 ** scale_exp).astype(np.float32)
+    vals[0] = np.float32(2.0 ** scale_exp * (1 + 2.0 ** -8))
+    for k in range(K):
+        a1[(k * 7) % M, k] = vals[k]
+        b1[k, (k * 11 + 2 + 64 * (k // M)) % N] = np.float32(2.0 ** 110)
+    want = a1.astype(np.float64) @ b1.astype(np.float64)
+    assert np.array_equal(run(a1, b1), want)
+    # and a later call with ordinary operands takes the split path again (the flag holds the earlier call's epoch)
+    a2, b2 = rng.standard_normal((M, K)).astype(np.float32), rng.standard_normal((K, N)).astype(np.float32)
+    assert rel_frobenius(run(a2, b2).ravel(), (a2.astype(np.float64) @ b2.astype(np.float64)).ravel()) <= 2e-6
 
 
 PERSISTENT = [  # op, dtA, bA, dtB, bB, out_dt, out_bias, M, N, K, batch, rows per reference launch
