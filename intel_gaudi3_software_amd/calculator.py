@@ -149,11 +149,13 @@ class HipCalculator:
         if rc != 0:
             raise MMEStackException(self._lib.mme_hip_last_error(None).decode(), rc)
         self._caller_stream = False
+        self._in_flight = []   # device operands of calls since the last synchronize()
 
     def close(self):
         if getattr(self, "_h", None) is not None and self._h.value:
-            self._lib.mme_hip_destroy(self._h)
+            self._lib.mme_hip_destroy(self._h)   # (waits for the stream)
             self._h = C.c_void_p()
+            self._in_flight = []
 
     def __del__(self):
         try:
@@ -214,6 +216,7 @@ class HipCalculator:
     # ---- extensions of the GPU path ------------------------------------------------------------------------------------
     def synchronize(self):
         self._check(self._lib.mme_hip_synchronize(self._h))
+        self._in_flight.clear()
 
     def stream(self):
         return self._lib.mme_hip_stream(self._h)
@@ -227,19 +230,18 @@ class HipCalculator:
 
     def _after_torch(self, *device_tensors):
         # the calculator's own stream does not synchronise with any other: make it wait (on the device) for the fills and
-        # copies that produced the operands on torch's current stream, and tell torch's allocator that the operands are in
-        # use on that stream, so that a temporary passed inline is not handed to the next allocation while a kernel still
-        # reads it.  Results may be consumed on torch's stream after synchronize().
+        # copies that produced the operands on torch's current stream, and keep the operands referenced until the next
+        # synchronize(), so that a temporary passed inline is not released to torch's allocator (and handed to the next
+        # allocation) while a kernel still reads it.  Results may be consumed on torch's stream after synchronize().
         if self._caller_stream:
             return
         import torch
-        own = torch.cuda.ExternalStream(self.stream())
         ev = torch.cuda.Event()
         ev.record()
-        own.wait_event(ev)
-        for t in device_tensors:
-            if t is not None and getattr(t, "is_cuda", False):
-                t.record_stream(own)
+        torch.cuda.ExternalStream(self.stream()).wait_event(ev)
+        self._in_flight.extend(t for t in device_tensors if t is not None and getattr(t, "is_cuda", False))
+        if len(self._in_flight) > 512:
+            self.synchronize()
 
     def setFp8SpecialsPolicy(self, policy):
         self._check(self._lib.mme_hip_set_fp8_specials_policy(self._h, policy))

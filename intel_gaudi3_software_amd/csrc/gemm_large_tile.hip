@@ -116,6 +116,8 @@ hipError_t launch_gemm_large_tile_conv_fp8(const GemmProblem& p, dim3 grid, hipS
 hipError_t launch_gemm_large_tile_fp8_at(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_fp8_at.hip
 hipError_t launch_gemm_large_tile_ragged(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged.hip
 hipError_t launch_gemm_large_tile_ragged_conv(const GemmProblem& p, dim3 grid, hipStream_t s); // gemm_large_tile_ragged_conv.hip
+hipError_t launch_gemm_large_tile_chk(const GemmProblem& p, dim3 grid, hipStream_t s);            // gemm_large_tile_chk.hip
+hipError_t launch_gemm_large_tile_persistent_chk(const GemmProblem& p, hipStream_t s);            // gemm_large_tile_persistent_chk.hip
 bool       gemm_large_tile_persistent_applicable(const GemmProblem& p);                      // gemm_large_tile_persistent.hip
 hipError_t launch_gemm_large_tile_persistent(const GemmProblem& p, hipStream_t s);
 
@@ -188,6 +190,14 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
     return true;
 }
 
+// fp8 problems that end up in gemm_fp8_fast_kernel or gemm_fp8_persistent_kernel (see launch_gemm_large_tile): plain views,
+// A k-contiguous, whole 256-row tiles
+bool gemm_large_tile_checks_operands(const GemmProblem& p)
+{
+    if (!(p.dtype == DT_FP8_143 || p.dtype == DT_FP8_152) || !gemm_large_tile_applicable(p)) return false;
+    return !large_tile_ragged(p) && p.tile_m != 128 && p.A.kind == VIEW_PLAIN && p.B.kind == VIEW_PLAIN && p.A.k_contig;
+}
+
 int gemm_fast_pick_tile_m(const GemmProblem& p, int num_cus)
 {
     GemmProblem q = p;
@@ -242,9 +252,11 @@ hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s)
     if (tm == 128) return launch_gemm_large_tile_128(p, grid, s);
     if (p.dtype == DT_FP16) return launch_gemm_large_tile_f16(p, grid, s);
     if (p.A.kind == VIEW_CONV && p.A.pix_is_f) return p.dtype == DT_BF16 ? launch_conv_bf16(p, grid, s) : launch_gemm_large_tile_conv_fp8(p, grid, s);
-    if (p.A.k_contig && gemm_large_tile_persistent_applicable(p)) return launch_gemm_large_tile_persistent(p, s);
+    if (p.A.k_contig && gemm_large_tile_persistent_applicable(p))
+        return p.chk && p.dtype != DT_BF16 ? launch_gemm_large_tile_persistent_chk(p, s) : launch_gemm_large_tile_persistent(p, s);
     if (p.dtype == DT_BF16) return launch_bf16(p, grid, s);
     if (!p.A.k_contig) return launch_gemm_large_tile_fp8_at(p, grid, s);
+    if (p.chk) return launch_gemm_large_tile_chk(p, grid, s);
     switch ((p.fmt_a & 1) | ((p.fmt_b & 1) << 1))
     {
         case 0: return launch_fmt<0>(p, grid, s);

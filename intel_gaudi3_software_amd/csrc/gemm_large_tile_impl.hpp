@@ -169,9 +169,15 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // a workgroup walks over tiles id, id + 256, ... of all batch elements.  Once the last fragments of a tile have left the
 // ring, the first four stages of the next tile are requested, and the epilogue of the finished tile (which stages its
 // stores in the 32 KiB of LDS behind the ring) runs while they arrive: pipeline fill and epilogue overlap.
-template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false>
+// CHK (fp8, AMODE 0, whole 256-row tiles): the kernel inspects the operand bytes on their way to the matrix cores for codes
+// that the hardware's fp8 formats read differently from Gaudi's (GemmProblem::chk_*) and raises the problem's flag when it
+// meets one.  Every 64-byte stage of an operand row is looked at by exactly one of the workgroups that read it (stage t of
+// the A rows by the tile column t mod tiles_n, of the B columns by the tile row t mod tiles_m), a few vector instructions
+// in the shadow of the matrix instructions, so a clean operand costs no extra pass over memory and no extra launch.
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
+    static_assert(!CHK || (ES == 1 && AMODE == 0 && TM == FBM && !RG), "operand checks: fp8, plain k-contiguous A, whole 256-row tiles");
     static_assert(!PERSIST || (AMODE == 0 && TM == FBM && !RG), "the persistent schedule: plain k-contiguous A, whole 256-row tiles");
     static_assert(TM == 256 || (TM == 128 && AMODE != 2), "the 128-row tile is not instantiated for plain f-contiguous A");
     static_assert(TM == 256 || ES == 2 || AMODE < 2, "fp8 operands that are contiguous along the tile's rows: 256-row tiles only");
@@ -188,12 +194,13 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     constexpr bool A_KC = AMODE < 2;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     warm_kernargs(g);
-    if (g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
+    if (!CHK && g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
 
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
     const int tiles_n = RG ? (g.N + FBN - 1) / FBN : g.N / FBN, tiles_m = (g.M + TM - 1) / TM;
     const int tiles_total = tiles_m * tiles_n;
-    int       m0 = 0, n0 = 0, b0 = 0, b1 = 0, b2 = 0;
+    int       m0 = 0, n0 = 0, b0 = 0, b1 = 0, b2 = 0, cur_tm = 0, cur_tn = 0;
+    uint32_t  chk_bad = 0; // CHK: bit 7 of a byte is set once a special code has been seen
     const long long lda = (A_KC ? g.A.stride_f : g.A.stride_k) * ES; // bytes between rows of the staged A tile
     const long long ldb = (B_KC ? g.B.stride_f : g.B.stride_k) * ES;
     const uint8_t*  A = nullptr;
@@ -221,6 +228,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         const long long b_off = b0 * g.B.batch_stride[0] + b1 * g.B.batch_stride[1] + b2 * g.B.batch_stride[2];
         m0 = tm * TM;
         n0 = tn * FBN;
+        cur_tm = tm;
+        cur_tn = tn;
         A = (const uint8_t*) g.A.base + a_off * ES;
         B = (const uint8_t*) g.B.base + b_off * ES;
     };
@@ -533,6 +542,18 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     if (LOADS) issue_a(u, t + FNST, slot);
 #define LB(u) \
     if (LOADS) issue_b(u, t + FNST, slot);
+#define CA(i) \
+    if (CHK && do_a) chk_frag(f.a[i], g.chk_mask_a, g.chk_add_a);
+#define CB(j) \
+    if (CHK && do_b) chk_frag(f.b[j], g.chk_mask_b, g.chk_add_b);
+    auto chk_frag = [&](const v8i& fr, uint32_t mask, uint32_t add) __attribute__((always_inline))
+    {
+#pragma unroll
+        for (int q = 0; q < 8; q += 2) chk_bad |= (((uint32_t) fr[q] & mask) + add) | (((uint32_t) fr[q + 1] & mask) + add);
+    };
+    // stages until this workgroup's next turn to look at the A rows / B columns of its tile (wavefronts with wn == 0 hold
+    // every A row of the tile between them, those with wm == 0 every B column)
+    int chk_ca = cur_tn, chk_cb = cur_tm;
     // One stage: 8 MFMAs; after the first one wait until stage t+1 has landed in every wavefront's view (WAITC leaves the
     // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
     // other wavefront on the SIMD covers the tail of that latency); request stage t+4 into the slot of stage t, whose
@@ -544,6 +565,14 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         constexpr bool RN = decltype(readnext)::value;
         const char*    st = lds + ((t + 1) % FNST) * STAGE;
         const int      slot = t % FNST;
+        bool           do_a = false, do_b = false;
+        if constexpr (CHK)
+        {
+            do_a = chk_ca == 0 && wn == 0 && g.chk_mask_a != 0;
+            do_b = chk_cb == 0 && wm == 0 && g.chk_mask_b != 0;
+            chk_ca = chk_ca == 0 ? tiles_n - 1 : chk_ca - 1;
+            chk_cb = chk_cb == 0 ? tiles_m - 1 : chk_cb - 1;
+        }
         MMA(0, 0);
         FENCE;
         if (RN)
@@ -555,13 +584,13 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         MMA(0, 1); FENCE;
         if constexpr (NI == 4)
         {
-            RA(0) LA(0) MMA(1, 0); FENCE;
+            CA(0) RA(0) LA(0) MMA(1, 0); FENCE;
             MMA(1, 1); FENCE;
-            RA(1) LA(1) MMA(2, 0); FENCE;
+            CA(1) RA(1) LA(1) MMA(2, 0); FENCE;
             MMA(2, 1); FENCE;
-            RA(2) LB(0) MMA(3, 0); FENCE;
-            RB(0) LB(1) MMA(3, 1); FENCE;
-            RA(3) RB(1) FENCE;
+            CA(2) RA(2) LB(0) MMA(3, 0); FENCE;
+            CB(0) RB(0) LB(1) MMA(3, 1); FENCE;
+            CA(3) CB(1) RA(3) RB(1) FENCE;
         }
         else
         {
@@ -592,6 +621,13 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #undef RB
 #undef LA
 #undef LB
+#undef CA
+#undef CB
+    if constexpr (CHK)
+    {
+        if (chk_bad & 0x80808080u) *const_cast<uint32_t*>((const uint32_t*) g.skip_flag) = g.skip_epoch;
+        chk_bad = 0;
+    }
 
     // ---- epilogue: alpha, per-column power of two, relu, cast, store (same conversion functions as the general kernel).
     // The matrix-core operands are swapped (B fragment first), so accumulator register v of lane l is output column

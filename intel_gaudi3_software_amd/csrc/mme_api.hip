@@ -466,15 +466,32 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         HIP_TRY(h, launch_gemm(g, h->stream));
         return MME_HIP_OK;
     }
-    // scan -> flag; native kernel runs when flag == 0; decode + bf16 kernel run when flag != 0
+    // the flag holds the epoch of the latest call that met such a code; the native kernel either finds them itself while it
+    // multiplies (the large-tile kernels that can) or is skipped when a scan launch in front of it found one; decode + bf16
+    // kernel run only when the flag holds this call's epoch, and then write the whole output
     if (int rc = ensure_flag(h)) return rc;
     uint32_t*      flag = (uint32_t*) h->flag.p;
-    const uint32_t epoch = ++h->specials_epoch; // the flag holds the epoch of the latest call whose scan found something
-    HIP_TRY(h, launch_fp8_special_scan2(flag, epoch, a_base, span_elements(ta), ta->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[0], b_base,
-                                        span_elements(tb), tb->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[1], h->stream));
+    const uint32_t epoch = ++h->specials_epoch;
     g.skip_flag = flag;
     g.skip_epoch = epoch;
     g.skip_if = 1; // native variant: skipped when the scan found something
+    if (gemm_large_tile_checks_operands(g))
+    {
+        g.chk = 1;
+        const mme_hip_tensor* t[2] = {ta, tb};
+        uint32_t              mask[2], add[2];
+        for (int i = 0; i < 2; i++)
+        {
+            // a byte b is special when (b & m) == m: m = the exponent field (kind 0) or all of 0x7F (kind 1: only 0x7F / 0xFF)
+            const uint32_t m = plan.scan_kind[i] < 0 ? 0u : (plan.scan_kind[i] == 1 ? 0x7Fu : (t[i]->dtype == MME_HIP_FP8_143 ? 0x78u : 0x7Cu));
+            mask[i] = m * 0x01010101u;
+            add[i] = m ? (0x80u - m) * 0x01010101u : 0u;
+        }
+        g.chk_mask_a = mask[0], g.chk_add_a = add[0], g.chk_mask_b = mask[1], g.chk_add_b = add[1];
+    }
+    else
+        HIP_TRY(h, launch_fp8_special_scan2(flag, epoch, a_base, span_elements(ta), ta->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[0], b_base,
+                                            span_elements(tb), tb->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[1], h->stream));
     HIP_TRY(h, launch_gemm(g, h->stream));
 
     const size_t na = span_elements(ta), nb = span_elements(tb);
@@ -486,6 +503,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
                                     (const uint8_t*) b_base, nb, tb->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) tb->fp_bias, tb->inf_nan_mode, flag,
                                     epoch, h->stream));
     GemmProblem g2 = g;
+    g2.chk = 0;
     g2.dtype = DT_BF16;
     g2.A.base = (const char*) da;
     g2.B.base = (const char*) db;

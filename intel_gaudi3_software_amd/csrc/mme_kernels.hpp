@@ -116,6 +116,12 @@ struct GemmProblem
     const uint32_t* skip_flag;
     int             skip_if;
     uint32_t        skip_epoch;
+    // chk != 0 (fp8 operands, large-tile kernels that have the variant, see gemm_large_tile_checks_operands): the launch never
+    // skips; instead the kernel looks at the operand bytes it multiplies and stores skip_epoch into *skip_flag when a byte b
+    // of operand A (B) has (b & chk_mask_a) + chk_add_a >= 0x80, i.e. a code the hardware's fp8 formats read differently
+    // (mask 0: that operand needs no check).  The caller then enqueues the exact fall-back behind it, predicated on the flag.
+    int             chk;
+    uint32_t        chk_mask_a, chk_add_a, chk_mask_b, chk_add_b; // the byte constants replicated over a 32-bit word
 };
 
 size_t     gemm_workspace_bytes(const GemmProblem& p);
@@ -127,6 +133,8 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s);
 bool       gemm_large_tile_applicable(const GemmProblem& p);
 int        gemm_fast_pick_split_k(const GemmProblem& p, int num_cus); // 0: the large-tile kernel does not take this problem
 hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s);
+// the kernel this problem takes can check its fp8 operands for special codes itself (GemmProblem::chk)
+bool       gemm_large_tile_checks_operands(const GemmProblem& p);
 
 // forward convolution fast path (conv_fwd_fast.hip): bf16, 3x3, 64 -> 64 channels, stride 1, padding 1, dense NHWC
 bool       conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int W, int H, int D, const int stride[4], const int dil[4],
