@@ -343,6 +343,26 @@ int mme_hip_batch_gemm_dev(mme_hip_handle          h,
                            int                     op,
                            const mme_hip_epilogue* epilogue);
 
+/*
+ * mme_hip_batch_gemm_dev for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels and bit-identical
+ * results, but every work space the call needs (split-k partial sums, the decoded operand copies and the flag cell of the
+ * fp8 / fp16 / tf32 / fp32 fall-backs) is taken from a static device array of MME_HIP_NOALLOC_SCRATCH_BYTES that each
+ * device holds from the moment the library's code is loaded there until the process ends; the call never calls hipMalloc,
+ * hipFree or an allocating library routine.  A problem whose work space does not fit returns MME_HIP_ENOMEM with the sizes
+ * in mme_hip_last_error (large fp8 operands in an inf/NaN mode the hardware formats lack need decoded copies for the
+ * fall-back: set MME_HIP_FP8_SPECIALS_ASSUME_NONE where that holds, or use mme_hip_batch_gemm_dev).  All handles of a
+ * device share that device's array: calls that overlap in time on one device race on it, so serialise them (one stream,
+ * or events between streams).
+ */
+#define MME_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
+int mme_hip_batch_gemm_dev_noalloc(mme_hip_handle          h,
+                                   const mme_hip_tensor*   out,
+                                   const mme_hip_tensor*   x,
+                                   const mme_hip_tensor*   w,
+                                   int                     op,
+                                   const mme_hip_epilogue* epilogue);
+
 /* doConvolution on device-resident tensors; epilogue as above.  dedw with a
  * split reduction uses workspace from the handle (allocated on first use). */
 int mme_hip_convolution_dev(mme_hip_handle             h,

@@ -144,6 +144,7 @@ def load_library():
     L.mme_hip_memory_write.argtypes = [vp, _TP, _TP, C.c_int, C.c_int, C.c_int]
     L.mme_hip_memory_write_dev.argtypes = [vp, _TP, _TP, C.c_int, C.c_int, C.c_int]
     L.mme_hip_batch_gemm_dev.argtypes = [vp, _TP, _TP, _TP, C.c_int, C.POINTER(Epilogue)]
+    L.mme_hip_batch_gemm_dev_noalloc.argtypes = [vp, _TP, _TP, _TP, C.c_int, C.POINTER(Epilogue)]
     L.mme_hip_convolution_dev.argtypes = [vp, _TP, _TP, _TP, _TP, C.POINTER(ConvParams), C.c_int, C.POINTER(Epilogue)]
     L.mme_hip_activation_dev.argtypes = [vp, _TP, _TP] + [C.c_int] * 6
     L.mme_hip_cast_from_fp32_dev.argtypes = [vp, vp, C.c_int, C.c_uint, C.c_int, vp, C.c_size_t, C.c_int, vp,

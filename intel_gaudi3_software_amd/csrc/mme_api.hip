@@ -3,9 +3,11 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <random>
 #include <string>
@@ -16,8 +18,20 @@
 
 using namespace mme;
 
+// Scratch memory of the entry point that allocates nothing (mme_hip_batch_gemm_dev_noalloc): one array per device, held from
+// the moment the library's code is loaded on that device until the process ends.  Bytes 0 .. 255 hold the flag cell of the
+// fp8 / split-operand fall-backs, the rest is handed out per call (split-k partial sums, decoded operand copies).  In host
+// code the array's name is only a stand-in: its device address is asked for once per device (mme_hip_create, with that
+// device current) and kept in g_scratch_ptr.
+static __device__ __align__(256) unsigned char scratch[MME_HIP_NOALLOC_SCRATCH_BYTES];
+
 namespace
 {
+constexpr int         MAX_DEVICES = 64;
+void*                 g_scratch_ptr[MAX_DEVICES];      // device address of `scratch` on each device, null until asked for
+std::atomic<uint32_t> g_scratch_epoch[MAX_DEVICES];    // epoch numbers of the flag cell in `scratch`: shared by every handle of a device
+std::mutex            g_scratch_mutex;
+
 thread_local std::string g_create_error = "";
 
 struct DeviceBuffer
@@ -61,6 +75,10 @@ struct mme_hip_calc
     DeviceBuffer          flag;      // one 32-bit cell: epoch number of the latest call whose operands held codes the hardware formats lack
     uint32_t              specials_epoch = 0; // epoch number of the latest call that scanned
     int                   fp8_specials_policy = 0;
+    // set for the duration of a call through the entry point that allocates nothing: every workspace comes out of the
+    // device's static scratch array (noalloc_used: bytes handed out so far in this call)
+    bool                  noalloc = false;
+    size_t                noalloc_used = 0;
 };
 
 namespace
@@ -89,6 +107,27 @@ int hip_fail(mme_hip_handle h, hipError_t e, const char* what)
         hipError_t e_ = (expr);                                   \
         if (e_ != hipSuccess) return hip_fail((h), e_, #expr);    \
     } while (0)
+
+// Work space of `bytes` for the current call: the handle's grow-only buffer `buf`, or, in a call that may not allocate, the
+// next piece of the device's static scratch array.
+int take_ws(mme_hip_handle h, DeviceBuffer& buf, size_t bytes, void** out)
+{
+    if (!h->noalloc)
+    {
+        HIP_TRY(h, buf.reserve(bytes));
+        *out = buf.p;
+        return MME_HIP_OK;
+    }
+    const size_t need = (bytes + 255) & ~(size_t) 255;
+    if (h->noalloc_used + need > (size_t) MME_HIP_NOALLOC_SCRATCH_BYTES)
+        return fail(h, MME_HIP_ENOMEM,
+                    "this call needs %zu more bytes of work space, the static scratch of the allocation-free entry point has %zu of %zu left; use "
+                    "mme_hip_batch_gemm_dev",
+                    need, (size_t) MME_HIP_NOALLOC_SCRATCH_BYTES - h->noalloc_used, (size_t) MME_HIP_NOALLOC_SCRATCH_BYTES);
+    *out = (unsigned char*) g_scratch_ptr[h->device] + h->noalloc_used;
+    h->noalloc_used += need;
+    return MME_HIP_OK;
+}
 
 int elem_size(int dt)
 {
@@ -255,13 +294,24 @@ void set_plain_view(OperandView& v, const void* base, long long stride_f, long l
     v.vec_ok = ok;
 }
 
-int ensure_flag(mme_hip_handle h)
+// The flag cell of this call and a fresh epoch number for it.  A call that may not allocate uses the cell at the start of the
+// device's static scratch array (zero when the code is loaded) with epoch numbers that every handle of the device draws
+// from one counter, so that a stale value of another handle's call never equals this call's number.
+int next_flag_epoch(mme_hip_handle h, uint32_t** flag, uint32_t* epoch)
 {
+    if (h->noalloc)
+    {
+        *flag = (uint32_t*) g_scratch_ptr[h->device];
+        *epoch = ++g_scratch_epoch[h->device];
+        return MME_HIP_OK;
+    }
     if (!h->flag.p)
     {
         HIP_TRY(h, h->flag.reserve(256));
         HIP_TRY(h, launch_fill_u32((uint32_t*) h->flag.p, 0u, 64, h->stream)); // epoch numbers start at 1
     }
+    *flag = (uint32_t*) h->flag.p;
+    *epoch = ++h->specials_epoch;
     return MME_HIP_OK;
 }
 
@@ -289,8 +339,9 @@ int plan_launch(mme_hip_handle h, GemmProblem& g)
     g.workspace = nullptr;
     if (g.split_k > 1)
     {
-        HIP_TRY(h, h->split_ws.reserve(gemm_workspace_bytes(g)));
-        g.workspace = (float*) h->split_ws.p;
+        void* ws = nullptr;
+        if (int rc = take_ws(h, h->split_ws, gemm_workspace_bytes(g), &ws)) return rc;
+        g.workspace = (float*) ws;
     }
     return MME_HIP_OK;
 }
@@ -354,10 +405,11 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
         part_elems[0] = part_elems[1] = 0;
     }
     const size_t fp32_copies = fp32_in ? 0 : na_pad + ((nb + 3) & ~(size_t) 3);
-    HIP_TRY(h, h->decode_ws.reserve((fp32_copies + 4) * 4 + (part_elems[0] + part_elems[1]) * 2));
-    float*    da = (float*) h->decode_ws.p;
+    void* decode_ws = nullptr;
+    if (int rc = take_ws(h, h->decode_ws, (fp32_copies + 4) * 4 + (part_elems[0] + part_elems[1]) * 2, &decode_ws)) return rc;
+    float*    da = (float*) decode_ws;
     float*    db = da + na_pad;
-    uint16_t* parts = (uint16_t*) ((float*) h->decode_ws.p + fp32_copies);
+    uint16_t* parts = (uint16_t*) ((float*) decode_ws + fp32_copies);
     const mme_hip_tensor* t[2] = {ta, tb};
     const void*           src[2] = {a_base, b_base};
     uint32_t*             flag = nullptr;
@@ -365,9 +417,7 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
     GemmProblem           g2 = g;
     if (two_part)
     {
-        if (int rc = ensure_flag(h)) return rc;
-        flag = (uint32_t*) h->flag.p;
-        epoch = ++h->specials_epoch;
+        if (int rc = next_flag_epoch(h, &flag, &epoch)) return rc;
         OperandView* v2[2] = {&g2.A, &g2.B};
         uint16_t*    dst = parts;
         for (int i = 0; i < 2; i++)
@@ -469,9 +519,9 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     // the flag holds the epoch of the latest call that met such a code; the native kernel either finds them itself while it
     // multiplies (the large-tile kernels that can) or is skipped when a scan launch in front of it found one; decode + bf16
     // kernel run only when the flag holds this call's epoch, and then write the whole output
-    if (int rc = ensure_flag(h)) return rc;
-    uint32_t*      flag = (uint32_t*) h->flag.p;
-    const uint32_t epoch = ++h->specials_epoch;
+    uint32_t* flag = nullptr;
+    uint32_t  epoch = 0;
+    if (int rc = next_flag_epoch(h, &flag, &epoch)) return rc;
     g.skip_flag = flag;
     g.skip_epoch = epoch;
     g.skip_if = 1; // native variant: skipped when the scan found something
@@ -496,8 +546,9 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
 
     const size_t na = span_elements(ta), nb = span_elements(tb);
     const size_t na_pad = (na + 7) & ~(size_t) 7;
-    HIP_TRY(h, h->decode_ws.reserve((na_pad + nb + 8) * 2));
-    uint16_t* da = (uint16_t*) h->decode_ws.p;
+    void* decode_ws = nullptr;
+    if (int rc = take_ws(h, h->decode_ws, (na_pad + nb + 8) * 2, &decode_ws)) return rc;
+    uint16_t* da = (uint16_t*) decode_ws;
     uint16_t* db = da + na_pad;
     HIP_TRY(h, launch_fp8_to_bf16_2(da, (const uint8_t*) a_base, na, ta->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) ta->fp_bias, ta->inf_nan_mode, db,
                                     (const uint8_t*) b_base, nb, tb->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) tb->fp_bias, tb->inf_nan_mode, flag,
@@ -589,6 +640,27 @@ int mme_hip_create(mme_hip_handle* out, int chip, int max_tensor_dims, int max_c
         return fail(nullptr, MME_HIP_EHIP, "no usable HIP device: %s", hipGetErrorString(e));
     }
     h->stream = h->own_stream;
+    if (h->device < 0 || h->device >= MAX_DEVICES)
+    {
+        const int dev = h->device;
+        mme_hip_destroy(h);
+        return fail(nullptr, MME_HIP_EHIP, "device index %d is beyond the %d devices this library keeps scratch addresses for", dev, MAX_DEVICES);
+    }
+    {
+        // the device address of this device's copy of the static scratch array (the current device is the handle's)
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[h->device])
+        {
+            void* p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p)
+            {
+                mme_hip_destroy(h);
+                return fail(nullptr, MME_HIP_EHIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+            }
+            g_scratch_ptr[h->device] = p;
+        }
+    }
     // LFSR registers and polynomial exactly as the reference seeds them (mme_reference_impl.cpp:146-170)
     h->lfsr.resize(lfsr_num_regs);
     for (uint32_t i = 0; i < lfsr_num_regs; i++) h->lfsr[i] = lfsr ? lfsr[i] : i + 2;
@@ -712,6 +784,25 @@ int mme_hip_batch_gemm_dev(mme_hip_handle h, const mme_hip_tensor* out, const mm
     g.epi.ld = out->strides[1];
     for (int d = 0; d < 3; d++) g.epi.batch_stride[d] = out->strides[d + 2];
     return run_contraction(h, g, x, w, x->data, w->data);
+}
+
+int mme_hip_batch_gemm_dev_noalloc(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, int op,
+                                   const mme_hip_epilogue* epi)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (!g_scratch_ptr[h->device]) return fail(h, MME_HIP_EHIP, "the static scratch array has no address on device %d", h->device);
+    // every work space request of this call is served from the static array; nothing below allocates or frees
+    struct Scope
+    {
+        mme_hip_handle h;
+        explicit Scope(mme_hip_handle h_) : h(h_)
+        {
+            h->noalloc = true;
+            h->noalloc_used = 256; // the flag cell
+        }
+        ~Scope() { h->noalloc = false; }
+    } scope(h);
+    return mme_hip_batch_gemm_dev(h, out, x, w, op, epi);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------
