@@ -216,6 +216,15 @@ int mme_hip_set_stream(mme_hip_handle h, void* hip_stream);
 int mme_hip_synchronize(mme_hip_handle h);
 
 /*
+ * Kernels whose wavefronts hand work to each other through counters in LDS (the 3x3 forward convolution) poll those counters
+ * a bounded number of times; a wavefront that runs out of polls records that in a status word and goes on, so every kernel
+ * ends, and mme_hip_synchronize (and the host-pointer entry points) then return MME_HIP_EHIP: the outputs since the last
+ * synchronisation are not valid.  This sets the bound (default 2^22 polls of about 64 clocks).  No counterpart in the
+ * reference; a host-side test uses a bound of zero to exercise the report.
+ */
+int mme_hip_set_wait_limit(mme_hip_handle h, unsigned polls);
+
+/*
  * clipFp / clipFpInfIn of the operand conversion, for the device-pointer contraction entry points (the host-pointer
  * ones take them per call).  On Gaudi3 only the tf32 flavour reads them: its operands are rounded from fp32 to tf32 on
  * entry and an overflow to infinity is clipped to the largest finite value when clip_fp is set (and, for an infinite

@@ -136,6 +136,7 @@ def load_library():
     L.mme_hip_stream.restype = vp
     L.mme_hip_set_stream.argtypes = [vp, vp]
     L.mme_hip_synchronize.argtypes = [vp]
+    L.mme_hip_set_wait_limit.argtypes = [vp, C.c_uint]
     L.mme_hip_set_fp8_specials_policy.argtypes = [vp, C.c_int]
     L.mme_hip_set_operand_clip.argtypes = [vp, C.c_int, C.c_int]
     L.mme_hip_batch_gemm.argtypes = [vp, _TP, _TP, _TP, C.c_int, C.c_int, C.c_int, C.c_int]

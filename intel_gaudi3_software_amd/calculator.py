@@ -243,6 +243,11 @@ class HipCalculator:
         if len(self._in_flight) > 512:
             self.synchronize()
 
+    def setWaitLimit(self, polls):
+        """Bound on the polls of a kernel's internal waits (mme_hip_set_wait_limit); a wait that runs out is reported by the
+        next synchronize()."""
+        self._check(self._lib.mme_hip_set_wait_limit(self._h, polls))
+
     def setFp8SpecialsPolicy(self, policy):
         self._check(self._lib.mme_hip_set_fp8_specials_policy(self._h, policy))
 

@@ -792,6 +792,40 @@ hipError_t launch_split_bf16(uint16_t* out, const void* in, int dtype, const Spl
     }
 }
 
+template<class T>
+__global__ __launch_bounds__(CAST_THREADS) void strided_copy_kernel(T* __restrict__ dst, const T* __restrict__ src, StridedCopyArgs a, size_t total)
+{
+    for (size_t i = (size_t) blockIdx.x * CAST_THREADS + threadIdx.x; i < total; i += (size_t) gridDim.x * CAST_THREADS)
+    {
+        size_t r = i, so = 0, d_o = 0;
+#pragma unroll
+        for (int d = 0; d < 5; d++)
+        {
+            const size_t c = r % a.sizes[d];
+            r /= a.sizes[d];
+            so += c * a.src_strides[d];
+            d_o += c * a.dst_strides[d];
+        }
+        dst[d_o] = src[so];
+    }
+}
+
+hipError_t launch_strided_copy(void* dst, const void* src, int elem_size, const StridedCopyArgs& a, hipStream_t s)
+{
+    size_t total = 1;
+    for (int d = 0; d < 5; d++) total *= a.sizes[d];
+    if (total == 0) return hipSuccess;
+    const int grid = grid_for(total, 1 << 16);
+    switch (elem_size)
+    {
+        case 1: hipLaunchKernelGGL((strided_copy_kernel<uint8_t>), dim3(grid), dim3(CAST_THREADS), 0, s, (uint8_t*) dst, (const uint8_t*) src, a, total); break;
+        case 2: hipLaunchKernelGGL((strided_copy_kernel<uint16_t>), dim3(grid), dim3(CAST_THREADS), 0, s, (uint16_t*) dst, (const uint16_t*) src, a, total); break;
+        case 4: hipLaunchKernelGGL((strided_copy_kernel<uint32_t>), dim3(grid), dim3(CAST_THREADS), 0, s, (uint32_t*) dst, (const uint32_t*) src, a, total); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s)
 {
     if (n == 0) return hipSuccess;

@@ -51,7 +51,26 @@ struct ConvFwdFastArgs
     int             B, H, W;
     int             rows_per_wg, rows_extra; // B * H output rows = gridDim.x * rows_per_wg + rows_extra (the first rows_extra workgroups take one more)
     GemmEpilogue    epi; // out = [B][H][W][64], ld = 64
+    // waits on LDS counters are bounded: after wait_limit polls a wavefront writes CF_GAVE_UP to *status (host-visible
+    // memory of the calculator) and goes on, so that a slip in the hand-over logic ends in an error report, not in a hang
+    uint32_t*       status;
+    uint32_t        wait_limit;
 };
+constexpr uint32_t CF_GAVE_UP = 0x57414954u; // "WAIT"
+
+__device__ __forceinline__ void cf_wait_for(uint32_t* counter, uint32_t target, uint32_t limit, uint32_t* status)
+{
+    uint32_t polls = 0;
+    while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target)
+    {
+        if (polls++ >= limit)
+        {
+            *status = CF_GAVE_UP;
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+}
 
 // 16 bytes per lane from global memory to LDS at lds_off + lane * 16 (lds_off is wave-uniform).  Inline assembly keeps
 // the request out of the compiler's memory model: it would otherwise order every later LDS read behind it.
@@ -106,12 +125,12 @@ __device__ __forceinline__ int cf_div(int n, int d)
 }
 
 // Barrier among the four wavefronts of a team: a counter in LDS that only grows.  (s_barrier would stop the other team
-// too.)  Every wavefront of the team reaches every barrier, so the spin always ends.
-__device__ __forceinline__ void cf_team_barrier(uint32_t* counter, uint32_t target, int lane)
+// too.)  Every wavefront of the team reaches every barrier, so the wait ends; it is bounded all the same (cf_wait_for).
+__device__ __forceinline__ void cf_team_barrier(uint32_t* counter, uint32_t target, int lane, uint32_t limit, uint32_t* status)
 {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     if (lane == 0) __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) __builtin_amdgcn_s_sleep(1);
+    cf_wait_for(counter, target, limit, status);
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
@@ -288,7 +307,7 @@ __global__ __launch_bounds__(512) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
                 __builtin_amdgcn_s_waitcnt(0x0F74);
             else
                 __builtin_amdgcn_s_waitcnt(0x0F70);
-            cf_team_barrier(counter, 4 * ++barriers, lane); // ... and the other three wavefronts' requests as well
+            cf_team_barrier(counter, 4 * ++barriers, lane, a.wait_limit, a.status); // ... and the other three wavefronts' requests as well
         }
         first = false;
         stores_in_flight = 0;
@@ -383,7 +402,7 @@ __global__ __launch_bounds__(512) void conv_fwd_fast_kernel(ConvFwdFastArgs a_by
         (void) h0_done;
         advance();
         if (row < row_end) advance();
-        cf_team_barrier(counter, 4 * ++barriers, lane);
+        cf_team_barrier(counter, 4 * ++barriers, lane, a.wait_limit, a.status);
         if (row < row_end) issue_halo(img, h0, nrows);
         if (tw >= ntiles) continue;
 
@@ -736,7 +755,7 @@ __global__ __launch_bounds__(512) void conv_fwd_resident_kernel(ConvFwdFastArgs 
         if (!landed && vtop_uniform((min(npx, (tile0 + 2) * 32) - 1) / W) + 3 > g0)
         {
             // every wavefront that raises the counter does so without waiting for anybody: the spin ends
-            while (__hip_atomic_load(ctrl + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < 4u) __builtin_amdgcn_s_sleep(1);
+            cf_wait_for(ctrl + 2, 4u, a.wait_limit, a.status);
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
             landed = true;
         }
@@ -896,7 +915,8 @@ bool conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int 
     return true;
 }
 
-hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int W, const GemmEpilogue& epi, int num_cus, hipStream_t s)
+hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int W, const GemmEpilogue& epi, int num_cus, uint32_t* status,
+                                uint32_t wait_limit, hipStream_t s)
 {
     static bool attr_done = false;
     const int   lds_bytes = CF_WT_BYTES + 2 * (CF_TR + 2) * (W + 2) * 128 + 16; // filter, one input tile per team, barrier counters
@@ -913,6 +933,8 @@ hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int 
     a.H = H;
     a.W = W;
     a.epi = epi;
+    a.status = status;
+    a.wait_limit = wait_limit;
     const long long rows = (long long) B * H;
     if (rows > 0x7fffffffLL) return hipErrorInvalidValue;
     const int grid = (int) std::min<long long>((rows + CF_TR - 1) / CF_TR, num_cus > 0 ? num_cus : 256);

@@ -11,6 +11,7 @@
 #include <new>
 #include <random>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "../../include/mme_hip.h"
@@ -72,6 +73,18 @@ struct mme_hip_calc
     std::string           error;
     DeviceBuffer          split_ws;  // split-k partial sums
     DeviceBuffer          decode_ws; // bf16 copies of fp8 operands the hardware formats cannot express
+    // host-pointer entry points: device copies of the call's tensors (grow-only, kept between calls) and two pinned bounce
+    // buffers with the events that say when the device has consumed / filled them
+    // one word of pinned host memory that kernels with bounded waits write when they give one up (read after a
+    // synchronisation), its device-side address, and the number of polls such a wait may take
+    uint32_t*             status_host = nullptr;
+    uint32_t*             status_dev = nullptr;
+    uint32_t              wait_limit = 1u << 22;
+    DeviceBuffer          stage_dev[3];
+    void*                 bounce[2] = {nullptr, nullptr};
+    hipEvent_t            bounce_ev[2] = {nullptr, nullptr};
+    DeviceBuffer          pack_ws[3]; // dense copies of convolution tensors whose strides the kernels cannot follow (weights, dy, output)
+    DeviceBuffer          stoch_ws;  // fp32 results of a contraction whose fused epilogue rounds stochastically
     DeviceBuffer          flag;      // one 32-bit cell: epoch number of the latest call whose operands held codes the hardware formats lack
     uint32_t              specials_epoch = 0; // epoch number of the latest call that scanned
     int                   fp8_specials_policy = 0;
@@ -213,8 +226,10 @@ int check_out_type(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_ep
         return fail(h, MME_HIP_EINVAL, "Unsupported type");
     if (is_fp16(out->dtype) && out->fp_bias > (out->dtype == MME_HIP_FP16 ? 31u : 63u))
         return fail(h, MME_HIP_EINVAL, "fp16 / ufp16 exponent bias exceeds the exponent field");
-    if (epi->rounding_mode == MME_HIP_RM_STOCHASTIC || epi->rounding_mode == MME_HIP_RM_STOCHASTIC_AND_NEAREST)
-        return fail(h, MME_HIP_EUNSUPPORTED, "stochastic rounding is not built for the fused epilogue");
+    {
+        const int rm = epi->rounding_mode;
+        if (!(rm == 0 || rm == 1 || rm == 2 || rm == 3 || rm == 4 || rm == 6 || rm == 7)) return fail(h, MME_HIP_EINVAL, "invalid rounding mode %d", rm);
+    }
     if (epi->scale_exp < -126 || epi->scale_exp > 126) return fail(h, MME_HIP_EINVAL, "scale exponent out of range");
     return MME_HIP_OK;
 }
@@ -593,6 +608,51 @@ int fill_epilogue(mme_hip_handle h, GemmEpilogue& e, const mme_hip_tensor* out, 
     (void) h;
     return MME_HIP_OK;
 }
+// after the stream has been synchronised: did a kernel give up one of its bounded waits since the last look?
+int check_status(mme_hip_handle h)
+{
+    const uint32_t code = *(volatile uint32_t*) h->status_host;
+    if (code == 0) return MME_HIP_OK;
+    *(volatile uint32_t*) h->status_host = 0;
+    return fail(h, MME_HIP_EHIP, "a kernel gave up a bounded wait on its workgroup's counters (code 0x%08x): the output of the calls since the last synchronisation is not valid", code);
+}
+
+bool stochastic_epilogue(const mme_hip_epilogue* epi)
+{
+    return epi && (epi->rounding_mode == MME_HIP_RM_STOCHASTIC || epi->rounding_mode == MME_HIP_RM_STOCHASTIC_AND_NEAREST);
+}
+} // namespace
+
+extern "C" int mme_hip_activation_dev(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* acc, int relu, int rm, int clip_fp,
+                                      int clip_inf_in, int flush_denorms, int stochastic_ftz);
+
+namespace
+{
+// A fused epilogue with a stochastic rounding mode.  The reference draws element i's random bits from LFSR register i % L
+// after i / L steps (convertToOutputDataType, mme_reference_impl.cpp:1153-1240), an order that belongs to the flat output
+// buffer, not to a tile walk; so the contraction writes its scaled (and rectified) fp32 results into a work space laid out
+// like the output, and the stochastic cast kernel of doActivation converts that, with the calculator's registers and in the
+// reference's order.  `contraction(tmp, epilogue)` runs the contraction into the fp32 tensor tmp.
+template<class F>
+int with_stochastic_epilogue(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_epilogue* epi, F&& contraction)
+{
+    mme_hip_tensor tmp = *out;
+    tmp.dtype = MME_HIP_FP32;
+    tmp.fp_bias = 0;
+    tmp.inf_nan_mode = MME_HIP_FULL_INF_NAN;
+    const size_t n = (size_t) span_elements(out);
+    void*        p = nullptr;
+    if (int rc = take_ws(h, h->stoch_ws, (n ? n : 1) * sizeof(float), &p)) return rc;
+    tmp.data = p;
+    // gaps between strided rows are converted too (the cast runs over the tensor's span): they hold zeros, as a freshly
+    // allocated accumulator tensor of the reference would
+    if (n != n_elements(out)) HIP_TRY(h, launch_fill_u32((uint32_t*) p, 0u, n, h->stream));
+    mme_hip_epilogue plain = *epi;
+    plain.rounding_mode = MME_HIP_RM_NEAREST_EVEN;
+    plain.clip_fp = plain.clip_inf_in = plain.flush_denorms = 0;
+    if (int rc = contraction(&tmp, &plain)) return rc;
+    return mme_hip_activation_dev(h, out, &tmp, 0, epi->rounding_mode, epi->clip_fp, epi->clip_inf_in, epi->flush_denorms, 0);
+}
 } // namespace
 
 // =====================================================================================================================
@@ -640,6 +700,17 @@ int mme_hip_create(mme_hip_handle* out, int chip, int max_tensor_dims, int max_c
         return fail(nullptr, MME_HIP_EHIP, "no usable HIP device: %s", hipGetErrorString(e));
     }
     h->stream = h->own_stream;
+    e = hipHostMalloc((void**) &h->status_host, 256, hipHostMallocMapped);
+    if (e == hipSuccess)
+    {
+        memset(h->status_host, 0, 256);
+        e = hipHostGetDevicePointer((void**) &h->status_dev, h->status_host, 0);
+    }
+    if (e != hipSuccess)
+    {
+        mme_hip_destroy(h);
+        return fail(nullptr, MME_HIP_EHIP, "no host-visible status word: %s", hipGetErrorString(e));
+    }
     if (h->device < 0 || h->device >= MAX_DEVICES)
     {
         const int dev = h->device;
@@ -684,6 +755,12 @@ void mme_hip_destroy(mme_hip_handle h)
         (void) hipStreamSynchronize(h->own_stream);
         (void) hipStreamDestroy(h->own_stream);
     }
+    if (h->status_host) (void) hipHostFree(h->status_host);
+    for (int i = 0; i < 2; i++)
+    {
+        if (h->bounce_ev[i]) (void) hipEventDestroy(h->bounce_ev[i]);
+        if (h->bounce[i]) (void) hipHostFree(h->bounce[i]);
+    }
     delete h;
 }
 
@@ -707,6 +784,13 @@ int mme_hip_synchronize(mme_hip_handle h)
 {
     if (!h) return MME_HIP_EINVAL;
     HIP_TRY(h, hipStreamSynchronize(h->stream));
+    return check_status(h);
+}
+
+int mme_hip_set_wait_limit(mme_hip_handle h, unsigned polls)
+{
+    if (!h) return MME_HIP_EINVAL;
+    h->wait_limit = polls;
     return MME_HIP_OK;
 }
 
@@ -740,6 +824,8 @@ int mme_hip_batch_gemm_dev(mme_hip_handle h, const mme_hip_tensor* out, const mm
     if (op < MME_HIP_OP_AB || op > MME_HIP_OP_ATBT) return fail(h, MME_HIP_EINVAL, "invalid bgemm op %d", op);
     if (int rc = check_operand_types(h, x, w)) return rc;
     if (int rc = check_out_type(h, out, epi)) return rc;
+    if (stochastic_epilogue(epi) && out->dtype != MME_HIP_FP32)
+        return with_stochastic_epilogue(h, out, epi, [&](const mme_hip_tensor* tmp, const mme_hip_epilogue* e) { return mme_hip_batch_gemm_dev(h, tmp, x, w, op, e); });
     for (int d = 2; d < 5; d++)
         if (!((x->sizes[d] == out->sizes[d] || x->sizes[d] == 1) && (w->sizes[d] == out->sizes[d] || w->sizes[d] == 1)))
             return fail(h, MME_HIP_EINVAL, "batch dims doesnt match !");
@@ -820,16 +906,33 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
         // weights are small; they are repacked into a workspace by one launch, as the reference does on the host
         if (int rc = check_tensor(h, w, "inputB")) return rc;
         uint64_t acc = 1;
+        bool     dense = true;
         for (int d = 0; d < 5; d++)
         {
-            if (w->sizes[d] > 1 && w->strides[d] != acc) return fail(h, MME_HIP_EUNSUPPORTED, "strided weight tensors are not built in this library");
+            dense = dense && !(w->sizes[d] > 1 && w->strides[d] != acc);
             acc *= w->sizes[d];
         }
-        const int es = elem_size(w->dtype);
-        HIP_TRY(h, h->weights_ws.reserve((size_t) acc * es + 16));
-        HIP_TRY(h, launch_repack_transposed_weights(h->weights_ws.p, w->data, es, w->sizes[0], w->sizes[1], w->sizes[2], (size_t) acc, h->stream));
+        const int   es = elem_size(w->dtype);
+        const void* w_dense = w->data;
+        void*       ws = nullptr;
+        if (!dense)
+        {
+            // strided weights: a dense copy first
+            if (int rc = take_ws(h, h->pack_ws[0], (size_t) acc * es + 16, &ws)) return rc;
+            StridedCopyArgs a;
+            uint32_t        run = 1;
+            for (int i = 0; i < 5; i++)
+            {
+                a.sizes[i] = w->sizes[i], a.src_strides[i] = w->strides[i], a.dst_strides[i] = run;
+                run *= w->sizes[i];
+            }
+            HIP_TRY(h, launch_strided_copy(ws, w->data, es, a, h->stream));
+            w_dense = ws;
+        }
+        if (int rc = take_ws(h, h->weights_ws, (size_t) acc * es + 16, &ws)) return rc;
+        HIP_TRY(h, launch_repack_transposed_weights(ws, w_dense, es, w->sizes[0], w->sizes[1], w->sizes[2], (size_t) acc, h->stream));
         mme_hip_tensor wr = *w;
-        wr.data = h->weights_ws.p;
+        wr.data = ws;
         wr.sizes[0] = w->sizes[1];
         wr.sizes[1] = w->sizes[0];
         acc = 1;
@@ -849,6 +952,11 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
     if (int rc = check_tensor(h, B, "inputB")) return rc;
     if (int rc = check_operand_types(h, A, B)) return rc;
     if (int rc = check_out_type(h, out, epi)) return rc;
+    if (stochastic_epilogue(epi) && out->dtype != MME_HIP_FP32)
+        return with_stochastic_epilogue(h, out, epi, [&](const mme_hip_tensor* tmp, const mme_hip_epilogue* e) {
+            // the output tensor also stands in the argument list under its role's name
+            return mme_hip_convolution_dev(h, tmp, op == MME_HIP_OP_DEDX ? tmp : x, op == MME_HIP_OP_DEDW ? tmp : w, op == MME_HIP_OP_FWD ? tmp : y, cp, op, e);
+        });
     for (int i = 0; i < 4; i++)
         if (cp->conv_stride[i] < 1 || cp->dilation[i] < 1) return fail(h, MME_HIP_EINVAL, "convolution stride and dilation must be positive");
 
@@ -865,13 +973,63 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
         return fail(h, MME_HIP_EINVAL, "convolution extents exceed 2^31");
     if (n_elements(out) == 0) return MME_HIP_OK;
 
-    // weights with one row pitch (rows of K output channels, one per (channel, tap)) and row-collapsible outputs keep the
-    // addressing linear
-    if (!rows_collapsible(wt)) return fail(h, MME_HIP_EUNSUPPORTED, "weight tensors whose rows do not share one pitch are not built in this library");
+    // The kernels address the weights as one matrix with a single row pitch (rows of K output channels, one per (channel,
+    // tap)), the output as rows of one pitch, and dedw's dy likewise.  A tensor whose strides do not collapse that way (the
+    // reference takes any strides, createBufferWith/WithoutStrides, mme_reference_impl.cpp:245-319) is contracted through a
+    // dense copy: inputs are gathered into one first, a result is computed densely and scattered into the caller's layout
+    // afterwards (only the tensor's own elements are written, what lies between them is left alone).
+    {
+        const mme_hip_tensor* w_in = op == MME_HIP_OP_DEDW ? nullptr : w;
+        const mme_hip_tensor* y_in = op == MME_HIP_OP_DEDW ? y : nullptr;
+        const bool            pack_w = w_in && !rows_collapsible(w_in), pack_y = y_in && !rows_collapsible(y_in), pack_out = !rows_collapsible(out);
+        if (pack_w || pack_y || pack_out)
+        {
+            auto dense_of = [](const mme_hip_tensor* t, void* data) {
+                mme_hip_tensor d = *t;
+                uint32_t       acc = 1;
+                for (int i = 0; i < 5; i++)
+                {
+                    d.strides[i] = acc;
+                    acc *= t->sizes[i];
+                }
+                d.data = data;
+                return d;
+            };
+            auto copy = [&](const mme_hip_tensor* dst, const mme_hip_tensor* src) {
+                StridedCopyArgs a;
+                for (int i = 0; i < 5; i++) a.sizes[i] = src->sizes[i], a.src_strides[i] = src->strides[i], a.dst_strides[i] = dst->strides[i];
+                return launch_strided_copy(dst->data, src->data, elem_size(src->dtype), a, h->stream);
+            };
+            mme_hip_tensor wd, yd, od;
+            void*          p = nullptr;
+            if (pack_w)
+            {
+                if (int rc = take_ws(h, h->pack_ws[0], (size_t) n_elements(w) * elem_size(w->dtype) + 16, &p)) return rc;
+                wd = dense_of(w, p);
+                HIP_TRY(h, copy(&wd, w));
+            }
+            if (pack_y)
+            {
+                if (int rc = take_ws(h, h->pack_ws[1], (size_t) n_elements(y) * elem_size(y->dtype) + 16, &p)) return rc;
+                yd = dense_of(y, p);
+                HIP_TRY(h, copy(&yd, y));
+            }
+            if (pack_out)
+            {
+                if (int rc = take_ws(h, h->pack_ws[2], (size_t) n_elements(out) * elem_size(out->dtype) + 16, &p)) return rc;
+                od = dense_of(out, p);
+            }
+            const mme_hip_tensor* o2 = pack_out ? &od : out;
+            const mme_hip_tensor* x2 = op == MME_HIP_OP_DEDX ? o2 : x;
+            const mme_hip_tensor* w2 = op == MME_HIP_OP_DEDW ? o2 : (pack_w ? &wd : w);
+            const mme_hip_tensor* y2 = op == MME_HIP_OP_FWD ? o2 : (pack_y ? &yd : y);
+            if (int rc = mme_hip_convolution_dev(h, o2, x2, w2, y2, cp, op, epi)) return rc;
+            if (pack_out) HIP_TRY(h, copy(out, &od));
+            return MME_HIP_OK;
+        }
+    }
     const long long w_ld = (long long) taps * C > 1 ? (long long) wt->strides[1] : Kc;
     if (w_ld < Kc) return fail(h, MME_HIP_EINVAL, "weight rows overlap");
-    if (!rows_collapsible(out)) return fail(h, MME_HIP_EUNSUPPORTED, "output tensors with non-collapsible row strides are not built");
-    if (op == MME_HIP_OP_DEDW && !rows_collapsible(y)) return fail(h, MME_HIP_EUNSUPPORTED, "dedw needs a row-collapsible dy tensor");
 
     const int es = elem_size(A->dtype);
     const int kv = 16 / es;
@@ -898,7 +1056,7 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
             GemmEpilogue e;
             if (int rc = fill_epilogue(h, e, out, epi)) return rc;
             e.ld = Kc;
-            HIP_TRY(h, launch_conv_fwd_fast(x->data, w->data, x->sizes[4], x->sizes[2], x->sizes[1], e, h->num_cus, h->stream));
+            HIP_TRY(h, launch_conv_fwd_fast(x->data, w->data, x->sizes[4], x->sizes[2], x->sizes[1], e, h->num_cus, h->status_dev, h->wait_limit, h->stream));
             return MME_HIP_OK;
         }
     }
@@ -1103,27 +1261,104 @@ int mme_hip_absmax_dev(mme_hip_handle h, float* out_absmax, const float* in, siz
 // ---------------------------------------------------------------------------------------------------------------------
 namespace
 {
+// Host memory <-> device memory for the reference-compatible entry points.  The caller's buffers are ordinary pageable
+// memory: they are moved through two pinned bounce buffers in chunks, the host-side copy of one chunk (a few threads)
+// running while the DMA engine moves the other, so that a large tensor travels at close to the link's rate.
+constexpr size_t BOUNCE_BYTES = (size_t) 16 << 20;
+constexpr size_t BOUNCE_THREAD_BYTES = (size_t) 2 << 20; // one host thread per this many bytes of a chunk, at most four
+
+void host_copy(void* dst, const void* src, size_t n)
+{
+    const size_t nt = std::min<size_t>(4, n / BOUNCE_THREAD_BYTES);
+    if (nt < 2)
+    {
+        memcpy(dst, src, n);
+        return;
+    }
+    std::vector<std::thread> workers;
+    const size_t             per = ((n / nt) + 4095) & ~(size_t) 4095;
+    for (size_t i = 1; i < nt; i++)
+    {
+        const size_t off = i * per, len = off >= n ? 0 : std::min(per, n - off);
+        if (len) workers.emplace_back([=] { memcpy((char*) dst + off, (const char*) src + off, len); });
+    }
+    memcpy(dst, src, std::min(per, n));
+    for (auto& w : workers) w.join();
+}
+
+int ensure_bounce(mme_hip_handle h)
+{
+    for (int i = 0; i < 2; i++)
+    {
+        if (!h->bounce[i]) HIP_TRY(h, hipHostMalloc(&h->bounce[i], BOUNCE_BYTES, hipHostMallocDefault));
+        if (!h->bounce_ev[i]) HIP_TRY(h, hipEventCreateWithFlags(&h->bounce_ev[i], hipEventDisableTiming));
+    }
+    return MME_HIP_OK;
+}
+
+int host_to_device(mme_hip_handle h, void* dst, const void* src, size_t bytes)
+{
+    if (int rc = ensure_bounce(h)) return rc;
+    int k = 0;
+    for (size_t off = 0; off < bytes; off += BOUNCE_BYTES, k++)
+    {
+        const int    slot = k & 1;
+        const size_t n = std::min(BOUNCE_BYTES, bytes - off);
+        if (k >= 2) HIP_TRY(h, hipEventSynchronize(h->bounce_ev[slot])); // the DMA of chunk k - 2 has read this buffer
+        host_copy(h->bounce[slot], (const char*) src + off, n);
+        HIP_TRY(h, hipMemcpyAsync((char*) dst + off, h->bounce[slot], n, hipMemcpyHostToDevice, h->stream));
+        HIP_TRY(h, hipEventRecord(h->bounce_ev[slot], h->stream));
+    }
+    // the bounce buffers are reused by the next transfer: it waits for these events first
+    for (int i = 0; i < 2 && i < k; i++) HIP_TRY(h, hipEventSynchronize(h->bounce_ev[(k - 1 - i) & 1]));
+    return MME_HIP_OK;
+}
+
+int device_to_host(mme_hip_handle h, void* dst, const void* src, size_t bytes)
+{
+    if (int rc = ensure_bounce(h)) return rc;
+    const size_t chunks = (bytes + BOUNCE_BYTES - 1) / BOUNCE_BYTES;
+    for (size_t k = 0; k <= chunks; k++)
+    {
+        if (k < chunks)
+        {
+            const size_t off = k * BOUNCE_BYTES, n = std::min(BOUNCE_BYTES, bytes - off);
+            HIP_TRY(h, hipMemcpyAsync(h->bounce[k & 1], (const char*) src + off, n, hipMemcpyDeviceToHost, h->stream));
+            HIP_TRY(h, hipEventRecord(h->bounce_ev[k & 1], h->stream));
+        }
+        if (k >= 1)
+        {
+            // chunk k - 1 has landed in its bounce buffer: hand it to the caller while chunk k is on its way
+            const size_t off = (k - 1) * BOUNCE_BYTES, n = std::min(BOUNCE_BYTES, bytes - off);
+            HIP_TRY(h, hipEventSynchronize(h->bounce_ev[(k - 1) & 1]));
+            host_copy((char*) dst + off, h->bounce[(k - 1) & 1], n);
+        }
+    }
+    return MME_HIP_OK;
+}
+
 struct Staged
 {
     mme_hip_tensor t;
-    DeviceBuffer   buf;
     void*          host = nullptr;
     size_t         bytes = 0;
 };
 
-int stage_in(mme_hip_handle h, Staged& s, const mme_hip_tensor* src, bool copy)
+// slot: which of the handle's three device-side staging buffers holds this tensor during the call
+int stage_in(mme_hip_handle h, Staged& s, int slot, const mme_hip_tensor* src, bool copy)
 {
     s.t = *src;
     s.host = src->data;
     s.bytes = (size_t) span_elements(src) * elem_size(src->dtype);
-    HIP_TRY(h, s.buf.reserve(s.bytes ? s.bytes : 16));
-    s.t.data = s.buf.p;
-    if (copy && s.bytes) HIP_TRY(h, hipMemcpyAsync(s.buf.p, s.host, s.bytes, hipMemcpyHostToDevice, h->stream));
+    HIP_TRY(h, h->stage_dev[slot].reserve(s.bytes ? s.bytes : 16));
+    s.t.data = h->stage_dev[slot].p;
+    if (copy && s.bytes) return host_to_device(h, s.t.data, s.host, s.bytes);
     return MME_HIP_OK;
 }
+// (returns with the bytes in the caller's buffer: the copy waits for the stream's work before it)
 int stage_out(mme_hip_handle h, Staged& s)
 {
-    if (s.bytes) HIP_TRY(h, hipMemcpyAsync(s.host, s.buf.p, s.bytes, hipMemcpyDeviceToHost, h->stream));
+    if (s.bytes) return device_to_host(h, s.host, s.t.data, s.bytes);
     return MME_HIP_OK;
 }
 bool has_gaps(const mme_hip_tensor* t) { return span_elements(t) != n_elements(t); }
@@ -1157,9 +1392,9 @@ int mme_hip_batch_gemm(mme_hip_handle h, const mme_hip_tensor* out, const mme_hi
     if (int rc = check_tensor(h, w, "w")) return rc;
     Staged so, sx, sw;
     // a strided output keeps the bytes between its rows: copy them in first
-    if (int rc = stage_in(h, so, out, has_gaps(out))) return rc;
-    if (int rc = stage_in(h, sx, x, true)) return rc;
-    if (int rc = stage_in(h, sw, w, true)) return rc;
+    if (int rc = stage_in(h, so, 0, out, has_gaps(out))) return rc;
+    if (int rc = stage_in(h, sx, 1, x, true)) return rc;
+    if (int rc = stage_in(h, sw, 2, w, true)) return rc;
     if (int rc = mme_hip_batch_gemm_dev(h, &so.t, &sx.t, &sw.t, op, nullptr)) return rc;
     if (int rc = stage_out(h, so)) return rc;
     HIP_TRY(h, hipStreamSynchronize(h->stream));
@@ -1172,24 +1407,28 @@ int mme_hip_convolution(mme_hip_handle h, const mme_hip_tensor* out, const mme_h
     (void) rm; // reaches only col2im's additions in the reference; all taps share one accumulator here
     if (!h) return MME_HIP_EINVAL;
     const OperandClipScope clip_scope(h, clip_fp, clip_fp_inf_in);
-    if (op != MME_HIP_OP_FWD && op != MME_HIP_OP_DEDX && op != MME_HIP_OP_DEDW)
-        return mme_hip_convolution_dev(h, out, x, w, y, cp, op, nullptr); // reports the error
-    const mme_hip_tensor* A = op == MME_HIP_OP_DEDX ? y : x;
+    // (any other operation is an error, and the device-pointer form reports it before it touches a tensor; never hand it a
+    // valid operation here: the tensors hold host pointers)
+    if (op != MME_HIP_OP_FWD && op != MME_HIP_OP_DEDX && op != MME_HIP_OP_DEDW && op != MME_HIP_OP_TRANSPOSED_DEDX)
+        return fail(h, MME_HIP_EINVAL, "invalid operation");
+    if (!out || !x || !w || !y) return fail(h, MME_HIP_EINVAL, "got null pointer");
+    const bool            dedx = op == MME_HIP_OP_DEDX || op == MME_HIP_OP_TRANSPOSED_DEDX; // the same roles, the weights laid out differently
+    const mme_hip_tensor* A = dedx ? y : x;
     const mme_hip_tensor* B = op == MME_HIP_OP_DEDW ? y : w;
     if (int rc = check_tensor(h, out, "output")) return rc;
     if (int rc = check_tensor(h, A, "inputA")) return rc;
     if (int rc = check_tensor(h, B, "inputB")) return rc;
     Staged so, sa, sb;
-    if (int rc = stage_in(h, so, out, has_gaps(out))) return rc;
-    if (int rc = stage_in(h, sa, A, true)) return rc;
-    if (int rc = stage_in(h, sb, B, true)) return rc;
-    const mme_hip_tensor* dx = op == MME_HIP_OP_DEDX ? &so.t : &sa.t;
+    if (int rc = stage_in(h, so, 0, out, has_gaps(out))) return rc;
+    if (int rc = stage_in(h, sa, 1, A, true)) return rc;
+    if (int rc = stage_in(h, sb, 2, B, true)) return rc;
+    const mme_hip_tensor* dx = dedx ? &so.t : &sa.t;
     const mme_hip_tensor* dw = op == MME_HIP_OP_DEDW ? &so.t : &sb.t;
-    const mme_hip_tensor* dy = op == MME_HIP_OP_FWD ? &so.t : (op == MME_HIP_OP_DEDX ? &sa.t : &sb.t);
+    const mme_hip_tensor* dy = op == MME_HIP_OP_FWD ? &so.t : (dedx ? &sa.t : &sb.t);
     if (int rc = mme_hip_convolution_dev(h, &so.t, dx, dw, dy, cp, op, nullptr)) return rc;
     if (int rc = stage_out(h, so)) return rc;
     HIP_TRY(h, hipStreamSynchronize(h->stream));
-    return MME_HIP_OK;
+    return check_status(h);
 }
 
 int mme_hip_activation(mme_hip_handle h, const mme_hip_tensor* out, const mme_hip_tensor* acc, int relu, int rm, int clip_fp, int clip_inf_in,
@@ -1199,8 +1438,8 @@ int mme_hip_activation(mme_hip_handle h, const mme_hip_tensor* out, const mme_hi
     if (int rc = check_tensor(h, out, "output")) return rc;
     if (int rc = check_tensor(h, acc, "acc")) return rc;
     Staged so, sa;
-    if (int rc = stage_in(h, so, out, true)) return rc;
-    if (int rc = stage_in(h, sa, acc, true)) return rc;
+    if (int rc = stage_in(h, so, 0, out, true)) return rc;
+    if (int rc = stage_in(h, sa, 1, acc, true)) return rc;
     if (int rc = mme_hip_activation_dev(h, &so.t, &sa.t, relu, rm, clip_fp, clip_inf_in, flush_denorms, stochastic_ftz)) return rc;
     if (int rc = stage_out(h, so)) return rc;
     if (relu)
@@ -1262,8 +1501,8 @@ int mme_hip_memory_write(mme_hip_handle h, const mme_hip_tensor* memory, const m
         o.strides[d] = memory->strides[d];
     }
     Staged sm, so;
-    if (int rc = stage_in(h, sm, memory, true)) return rc;
-    if (int rc = stage_in(h, so, &o, true)) return rc;
+    if (int rc = stage_in(h, sm, 0, memory, true)) return rc;
+    if (int rc = stage_in(h, so, 1, &o, true)) return rc;
     if (int rc = mme_hip_memory_write_dev(h, &sm.t, &so.t, reduction_op, reduction_rm, clip_fp)) return rc;
     if (int rc = stage_out(h, sm)) return rc;
     HIP_TRY(h, hipStreamSynchronize(h->stream));

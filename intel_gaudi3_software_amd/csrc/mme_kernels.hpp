@@ -30,6 +30,15 @@ hipError_t launch_repack_transposed_weights(void* out, const void* in, int elem_
 // zero, 2 up, 3 down)
 hipError_t launch_memory_write_reduce(void* memory, const void* mme_out, int dtype, size_t n, int op, int rm, int clip, hipStream_t s);
 hipError_t launch_relu_inplace(float* x, size_t n, hipStream_t s);
+// copies the logical elements of a 5-d tensor between two layouts: element (i0 .. i4) from src + sum i_d * src_strides[d] to
+// dst + sum i_d * dst_strides[d] (strides in elements of elem_size bytes); used to make a dense copy of a tensor whose
+// strides the contraction kernels cannot follow, and to write a dense result back into such a tensor
+struct StridedCopyArgs
+{
+    uint32_t sizes[5];
+    uint32_t src_strides[5], dst_strides[5];
+};
+hipError_t launch_strided_copy(void* dst, const void* src, int elem_size, const StridedCopyArgs& a, hipStream_t s);
 // fp32 words -> the same words rounded to tf32 (nearest even, 10 mantissa bits), out of place
 hipError_t launch_round_to_tf32(void* out, const void* in, size_t n, int clip, int clip_inf_in, hipStream_t s, const uint32_t* run_flag = nullptr,
                                 uint32_t run_epoch = 0);
@@ -139,7 +148,9 @@ bool       gemm_large_tile_checks_operands(const GemmProblem& p);
 // forward convolution fast path (conv_fwd_fast.hip): bf16, 3x3, 64 -> 64 channels, stride 1, padding 1, dense NHWC
 bool       conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int W, int H, int D, const int stride[4], const int dil[4],
                                     const int pad[4], bool dense);
-hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int W, const GemmEpilogue& epi, int num_cus, hipStream_t s);
+// status: host-visible word that a kernel sets when it gives up a bounded wait (after wait_limit polls)
+hipError_t launch_conv_fwd_fast(const void* x, const void* w, int B, int H, int W, const GemmEpilogue& epi, int num_cus, uint32_t* status,
+                                uint32_t wait_limit, hipStream_t s);
 
 // flags every exponent-all-ones code of an fp8 buffer (inf / NaN in Gaudi's full mode, finite for the hardware's
 // e4m3): *flag |= 1.  mask_kind 0: any code with all exponent bits set; 1: only 0x7F / 0xFF.

@@ -65,6 +65,113 @@ def test_conv_vs_oracle(calc, orc, case, dt, bias, op):
     assert np.all(got[want == 0] == 0) or op != abi.OP_DEDX
 
 
+def _odd_strides(sizes, pads, order):
+    """Element strides of a tensor whose dimensions 1 .. 4 lie in memory in the given order, each padded by pads[d] extra
+    entries: rows that do not collapse to one pitch."""
+    strides = [1, 0, 0, 0, 0]
+    run = sizes[0] + pads[0]
+    for d in order:
+        strides[d] = run
+        run *= sizes[d] + pads[d]
+    return strides, run
+
+
+@pytest.mark.parametrize("op", [abi.OP_FWD, abi.OP_DEDX, abi.OP_DEDW, abi.OP_TRANSPOSED_DEDX])
+@pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP8_152, 15)])
+@pytest.mark.parametrize("device", [False, True])
+def test_conv_tensors_with_arbitrary_strides(calc, orc, op, dt, bias, device):
+    """Weights, activations, gradients and outputs whose dimensions are padded and stored in another order (rows without a
+    common pitch): the reference follows any strides (createBufferWith/WithoutStrides, mme_reference_impl.cpp:245-319).
+    Every logical element against the oracle reading the same buffers; what lies between the output's elements keeps its
+    previous contents."""
+    import torch
+    rng = np.random.default_rng(300 + op)
+    C, K, W, H, D, B, S, R, Q = 24, 40, 7, 6, 3, 2, 3, 2, 2
+    pad, st, dil = (1, 0, 1), (1, 1, 1), (1, 1, 1)
+    Wo, Ho, Do = _osz(W, S, pad[0], st[0], dil[0]), _osz(H, R, pad[1], st[1], dil[1]), _osz(D, Q, pad[2], st[2], dil[2])
+    xs, ys = [C, W, H, D, B], [K, Wo, Ho, Do, B]
+    ws = [C, K, S, R, Q] if op == abi.OP_TRANSPOSED_DEDX else [K, C, S, R, Q]
+    (sx, nx), (sw, nw), (sy, ny) = _odd_strides(xs, [3, 1, 0, 2, 0], [2, 1, 4, 3]), _odd_strides(ws, [5, 2, 1, 0, 1], [3, 1, 2, 4]), \
+        _odd_strides(ys, [1, 0, 2, 1, 1], [1, 3, 2, 4])
+    x, w, y = random_operand(rng, dt, nx, orc, bias), random_operand(rng, dt, nw, orc, bias, scale=0.3), random_operand(rng, dt, ny, orc, bias, scale=0.5)
+    osz, so, no = {abi.OP_FWD: (ys, sy, ny), abi.OP_DEDX: (xs, sx, nx), abi.OP_TRANSPOSED_DEDX: (xs, sx, nx), abi.OP_DEDW: (ws, sw, nw)}[op]
+    want = np.full(no, 7.0, np.float32)
+    p = abi.make_conv_params(3, pad, st, dil)
+    dx, dw, dy, do = desc(x, xs, dt, bias, strides=sx), desc(w, ws, dt, bias, strides=sw), desc(y, ys, dt, bias, strides=sy), desc(want, osz, abi.FP32, strides=so)
+    assert orc.orc_convolution(A(do), A(dx), A(dw), A(dy), A(p), op, 0) == 0, orc.orc_last_error()
+    cp = ConvolutionParams(3, list(pad) + [0], list(st) + [1], list(dil) + [1])
+    if device:
+        conv = (lambda a: torch.from_numpy(a.view(np.int16) if a.dtype.itemsize == 2 else a).cuda())
+        to = torch.full((no,), 7.0, dtype=torch.float32, device="cuda")
+        calc.doConvolution(MmeSimTensor(osz, 5, abi.FP32, to, strides=so), MmeSimTensor(xs, 5, dt, conv(x), bias, strides=sx),
+                           MmeSimTensor(ws, 5, dt, conv(w), bias, strides=sw), MmeSimTensor(ys, 5, dt, conv(y), bias, strides=sy), cp, op)
+        calc.synchronize()
+        got = to.cpu().numpy()
+    else:
+        got = np.full(no, 7.0, np.float32)
+        calc.doConvolution(MmeSimTensor(osz, 5, abi.FP32, got, strides=so), MmeSimTensor(xs, 5, dt, x, bias, strides=sx),
+                           MmeSimTensor(ws, 5, dt, w, bias, strides=sw), MmeSimTensor(ys, 5, dt, y, bias, strides=sy), cp, op)
+    # the tensor's own elements
+    idx = np.zeros(osz[::-1], np.int64)
+    for d, (n, stv) in enumerate(zip(osz, so)):
+        shape = [1] * 5
+        shape[4 - d] = n
+        idx = idx + (np.arange(n, dtype=np.int64) * stv).reshape(shape)
+    idx = idx.ravel()
+    assert rel_frobenius(got[idx], want[idx]) <= TOL[dt] and np.any(want[idx] != 7.0)
+    rest = np.ones(no, bool)
+    rest[idx] = False
+    assert np.all(got[rest] == 7.0)
+
+
+def test_conv_fwd_bounded_waits_report_instead_of_hanging(orc):
+    """The 3 x 3 forward kernels hand rows between wavefronts through counters in LDS and poll them a bounded number of
+    times.  With the bound forced to zero from the host a wavefront that has to wait at all gives up at once: the kernel
+    still ends normally and the next synchronize() reports it; with the bound restored the same call is right again.  Both
+    forms of the kernel: the one that keeps a workgroup's rows resident in LDS and the two-team one."""
+    import torch
+    from intel_gaudi3_software_amd import HipCalculator
+    from intel_gaudi3_software_amd.calculator import MMEStackException
+    from helpers import bf16_bits_to_f32, to_bf16_bits
+    rng = np.random.default_rng(55)
+    calc = HipCalculator()
+    gave_up = []
+    try:
+        for B, H, W in [(8, 56, 56), (256, 56, 56)]:
+            Cc = Kk = 64
+            xs, ws, ys = [Cc, W, H, 1, B], [Kk, Cc, 3, 3, 1], [Kk, W, H, 1, B]
+            x = to_bf16_bits(np.maximum(rng.standard_normal(int(np.prod(xs))), 0).astype(np.float32))
+            w = to_bf16_bits((rng.standard_normal(int(np.prod(ws))) * 0.06).astype(np.float32))
+            tx, tw = torch.from_numpy(x.view(np.int16)).cuda(), torch.from_numpy(w.view(np.int16)).cuda()
+            ty = torch.zeros(int(np.prod(ys)), dtype=torch.float32, device="cuda")
+            X, Wt, Y = MmeSimTensor(xs, 5, abi.BF16, tx), MmeSimTensor(ws, 5, abi.BF16, tw), MmeSimTensor(ys, 5, abi.FP32, ty)
+            cp = ConvolutionParams(2, [1, 1, 0, 0])
+            calc.setWaitLimit(0)
+            print("bounded waits: limit 0,", B, H, W, flush=True)
+            calc.doConvolution(Y, X, Wt, Y, cp, abi.OP_FWD)
+            try:
+                calc.synchronize()
+                gave_up.append(False)
+            except MMEStackException as e:
+                assert "bounded wait" in str(e) and e.status == abi.EHIP
+                gave_up.append(True)
+            calc.setWaitLimit(1 << 22)
+            print("bounded waits: limit restored,", B, H, W, flush=True)
+            calc.doConvolution(Y, X, Wt, Y, cp, abi.OP_FWD)
+            calc.synchronize()   # no report this time
+            got = ty.cpu().numpy().reshape(B, H * W * Kk)
+            b = B - 1
+            xb = np.ascontiguousarray(x[b * H * W * Cc:(b + 1) * H * W * Cc])
+            want = np.zeros(H * W * Kk, np.float32)
+            p = abi.make_conv_params(2, (1, 1, 0), (1, 1, 1), (1, 1, 1))
+            dx, dw, do = desc(xb, [Cc, W, H, 1, 1], abi.BF16), desc(w, ws, abi.BF16), desc(want, [Kk, W, H, 1, 1], abi.FP32)
+            assert orc.orc_convolution(A(do), A(dx), A(dw), A(do), A(p), abi.OP_FWD, 0) == 0
+            assert rel_frobenius(got[b], want) <= 1e-4
+    finally:
+        calc.close()
+    assert any(gave_up), "no wavefront ever had to wait: the report path was not exercised"
+
+
 def test_conv_adjoint_identities(calc, orc):
     """<dY, fwd(X, W)> = <dedx(dY, W), X> = <dedw(X, dY), W> on a shape too large for the oracle to do quickly."""
     import torch
