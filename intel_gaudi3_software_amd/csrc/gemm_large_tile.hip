@@ -198,6 +198,11 @@ bool gemm_large_tile_checks_operands(const GemmProblem& p)
     return !large_tile_ragged(p) && p.tile_m != 128 && p.A.kind == VIEW_PLAIN && p.B.kind == VIEW_PLAIN && p.A.k_contig;
 }
 
+bool gemm_large_tile_takes_mfma_scale(const GemmProblem& p)
+{
+    return gemm_large_tile_checks_operands(p) && !p.chk && !(p.A.k_contig && gemm_large_tile_persistent_applicable(p));
+}
+
 int gemm_fast_pick_tile_m(const GemmProblem& p, int num_cus)
 {
     GemmProblem q = p;

@@ -123,25 +123,30 @@ __device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int w
 
 #define FENCE __builtin_amdgcn_sched_barrier(0)
 
+// s_waitcnt immediate that waits until at most n of this wavefront's memory requests are outstanding and leaves the other
+// counters alone (gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14)
+constexpr int vm_wait(int n) { return 0x0F70 | (n & 15) | ((n >> 4) << 14); }
+
 // The problem description is read in place from the kernarg segment, field by field where the code needs it: every 64-byte
 // line touched for the first time (tile set-up, gather set-up, epilogue) would be a miss of its own, one memory latency
 // each, in series.  One scalar load per line up front takes all those misses at once.
 __device__ __forceinline__ void warm_kernargs(KARG GemmProblem& g)
 {
-    static_assert(sizeof(GemmProblem) <= 640, "one load per 64-byte line of the problem description");
-    uint32_t t0, t1, t2, t3, t4, t5, t6, t7, t8, t9;
-    asm volatile("s_load_dword %0, %10, 0x0\n\t"
-                 "s_load_dword %1, %10, 0x40\n\t"
-                 "s_load_dword %2, %10, 0x80\n\t"
-                 "s_load_dword %3, %10, 0xc0\n\t"
-                 "s_load_dword %4, %10, 0x100\n\t"
-                 "s_load_dword %5, %10, 0x140\n\t"
-                 "s_load_dword %6, %10, 0x180\n\t"
-                 "s_load_dword %7, %10, 0x1c0\n\t"
-                 "s_load_dword %8, %10, 0x200\n\t"
-                 "s_load_dword %9, %10, 0x240\n\t"
+    static_assert(sizeof(GemmProblem) > 640 && sizeof(GemmProblem) <= 704, "one load per 64-byte line of the problem description");
+    uint32_t t0, t1, t2, t3, t4, t5, t6, t7, t8, t9, t10;
+    asm volatile("s_load_dword %0, %11, 0x0\n\t"
+                 "s_load_dword %1, %11, 0x40\n\t"
+                 "s_load_dword %2, %11, 0x80\n\t"
+                 "s_load_dword %3, %11, 0xc0\n\t"
+                 "s_load_dword %4, %11, 0x100\n\t"
+                 "s_load_dword %5, %11, 0x140\n\t"
+                 "s_load_dword %6, %11, 0x180\n\t"
+                 "s_load_dword %7, %11, 0x1c0\n\t"
+                 "s_load_dword %8, %11, 0x200\n\t"
+                 "s_load_dword %9, %11, 0x240\n\t"
+                 "s_load_dword %10, %11, 0x280\n\t"
                  "s_waitcnt lgkmcnt(0)"
-                 : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9)
+                 : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8), "=&s"(t9), "=&s"(t10)
                  : "s"(&g)
                  : "memory");
 }
@@ -174,9 +179,13 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // meets one.  Every 64-byte stage of an operand row is looked at by exactly one of the workgroups that read it (stage t of
 // the A rows by the tile column t mod tiles_n, of the B columns by the tile row t mod tiles_m), a few vector instructions
 // in the shadow of the matrix instructions, so a clean operand costs no extra pass over memory and no extra launch.
-template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false>
+// NST: stages of the ring (default 4).  What a compute unit can draw from L2 / memory is the bytes it has in flight divided
+// by the latency, so a kernel whose stages are small (the 128-row tile: 24 KiB) keeps more of them in flight: six stages,
+// 144 KiB.  The reduction then has to be at least NST stages long.
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
+    static_assert(NST >= 4 && NST <= 6 && (!PERSIST || NST == FNST), "ring depth");
     static_assert(!CHK || (ES == 1 && AMODE == 0 && TM == FBM && !RG), "operand checks: fp8, plain k-contiguous A, whole 256-row tiles");
     static_assert(!PERSIST || (AMODE == 0 && TM == FBM && !RG), "the persistent schedule: plain k-contiguous A, whole 256-row tiles");
     static_assert(TM == 256 || (TM == 128 && AMODE != 2), "the 128-row tile is not instantiated for plain f-contiguous A");
@@ -466,7 +475,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     // fragment registers, which happens one step before the stage is multiplied
     auto issue_prologue = [&]() __attribute__((always_inline))
     {
-        for (int t = 0; t < FNST; t++)
+        for (int t = 0; t < NST; t++)
         {
 #pragma unroll
             for (int u = 0; u < 2; u++)
@@ -480,7 +489,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     for (int walk_it = 0;;) // (one pass unless PERSIST)
     {
     // s_waitcnt immediate (gfx9): vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-    if (!PERSIST || walk_it == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (3 * NREQ)); // three stages may still be in flight: stage 0 has landed
+    if (!PERSIST || walk_it == 0) __builtin_amdgcn_s_waitcnt(vm_wait((NST - 1) * NREQ)); // all stages but the first may still be in flight: stage 0 has landed
     else
     {
         // a later tile: its four stages were requested before the previous tile's epilogue, whose stores share the counter
@@ -507,10 +516,20 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #pragma unroll
     for (int j = 0; j < 2; j++) read_b(f, j, lds);
 
+    constexpr bool MSCALE = ES == 1 && AMODE == 0 && TM == FBM && !RG && !PERSIST && !CHK;
+    const int      mfma_scale_a = 127 + (MSCALE ? g.epi.mfma_scale_exp : 0);
     auto mma = [&](int i, int j) __attribute__((always_inline))
     {
         if constexpr (ES == 1)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
+        {
+            // the block-scale operands are exponents (2^(byte - 127), byte 0 of the register): the first carries the
+            // epilogue's power-of-two factor when the host folded it in, the second is 2^0
+            // (only in the plain instance, see gemm_large_tile_takes_mfma_scale: with the scale operands the register allocator
+            // spills accumulators in the instances that walk over tiles or check their operands)
+            if constexpr (!MSCALE) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, mfma_scale_a, 0, 127);
+        }
         else
         {
             union
@@ -539,21 +558,33 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #define RB(j) \
     if (RN) read_b(f, j, st);
 #define LA(u) \
-    if (LOADS) issue_a(u, t + FNST, slot);
+    if (LOADS) issue_a(u, t + NST, slot);
 #define LB(u) \
-    if (LOADS) issue_b(u, t + FNST, slot);
+    if (LOADS) issue_b(u, t + NST, slot);
 #define CA(i) \
-    if (CHK && do_a) chk_frag(f.a[i], g.chk_mask_a, g.chk_add_a);
+    if (CHK && do_a && wn == i) chk_frag(f.a[i], chk_ma, chk_aa);
 #define CB(j) \
-    if (CHK && do_b) chk_frag(f.b[j], g.chk_mask_b, g.chk_add_b);
+    if (CHK && do_b && wm == j) chk_frag(f.b[j], chk_mb, chk_ab);
     auto chk_frag = [&](const v8i& fr, uint32_t mask, uint32_t add) __attribute__((always_inline))
     {
 #pragma unroll
         for (int q = 0; q < 8; q += 2) chk_bad |= (((uint32_t) fr[q] & mask) + add) | (((uint32_t) fr[q + 1] & mask) + add);
     };
-    // stages until this workgroup's next turn to look at the A rows / B columns of its tile (wavefronts with wn == 0 hold
-    // every A row of the tile between them, those with wm == 0 every B column)
+    // stages until this workgroup's next turn to look at the A rows / B columns of its tile.  The four wavefronts with the same
+    // wm hold the same four A fragments and take one each (fragment i by the wavefront with wn == i); the two wavefronts with
+    // the same wn hold the same two B fragments and take one each: the work of a turn is spread evenly over the SIMDs
     int chk_ca = cur_tn, chk_cb = cur_tm;
+    // the constants of the check, read from the kernel arguments once and pinned in scalar registers: a read inside a step
+    // would wait on the counter that the step's LDS reads share
+    uint32_t chk_ma = 0, chk_aa = 0, chk_mb = 0, chk_ab = 0;
+    bool     chk_a_mine = false, chk_b_mine = false;
+    if constexpr (CHK)
+    {
+        chk_ma = g.chk_mask_a, chk_aa = g.chk_add_a, chk_mb = g.chk_mask_b, chk_ab = g.chk_add_b;
+        asm volatile("" : "+s"(chk_ma), "+s"(chk_aa), "+s"(chk_mb), "+s"(chk_ab));
+        chk_a_mine = chk_ma != 0;
+        chk_b_mine = chk_mb != 0;
+    }
     // One stage: 8 MFMAs; after the first one wait until stage t+1 has landed in every wavefront's view (WAITC leaves the
     // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
     // other wavefront on the SIMD covers the tail of that latency); request stage t+4 into the slot of stage t, whose
@@ -563,13 +594,13 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         constexpr int  WAITC = decltype(waitc)::value;
         constexpr bool LOADS = decltype(loads)::value;
         constexpr bool RN = decltype(readnext)::value;
-        const char*    st = lds + ((t + 1) % FNST) * STAGE;
-        const int      slot = t % FNST;
+        const char*    st = lds + ((t + 1) % NST) * STAGE;
+        const int      slot = t % NST;
         bool           do_a = false, do_b = false;
         if constexpr (CHK)
         {
-            do_a = chk_ca == 0 && wn == 0 && g.chk_mask_a != 0;
-            do_b = chk_cb == 0 && wm == 0 && g.chk_mask_b != 0;
+            do_a = chk_ca == 0 && chk_a_mine;
+            do_b = chk_cb == 0 && chk_b_mine;
             chk_ca = chk_ca == 0 ? tiles_n - 1 : chk_ca - 1;
             chk_cb = chk_cb == 0 ? tiles_m - 1 : chk_cb - 1;
         }
@@ -600,22 +631,45 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             RA(1) RB(1) LB(1) FENCE;
         }
     };
-    using W8 = std::integral_constant<int, 0x0F70 | (2 * NREQ)>; // two stages of this wavefront's requests may still be in flight
-    using W4 = std::integral_constant<int, 0x0F70 | NREQ>;       // one stage
-    using W0 = std::integral_constant<int, 0x0F70>;              // vmcnt(0)
+    // at the wait of step t the stages t+1 .. t+NST-1 have been requested; stage t+1 is needed, so the younger NST-2 stages of
+    // this wavefront's requests may stay in flight
+    using WM = std::integral_constant<int, vm_wait((NST - 2) * NREQ)>;
     using T = std::true_type;
     using F = std::false_type;
     int t = 0;
-    for (; t + 5 <= nk; t += 2) // steps 0 .. nk-5 request stages 4 .. nk-1
+    for (; t + NST + 1 < nk; t += 2) // steps 0 .. nk-NST-1 request stages NST .. nk-1
     {
-        step(t, W8 {}, T {}, T {});
-        step(t + 1, W8 {}, T {}, T {});
+        step(t, WM {}, T {}, T {});
+        step(t + 1, WM {}, T {}, T {});
     }
-    // t == nk - 4 (nk is even and >= 6): everything has been requested
-    step(t, W8 {}, F {}, T {});     // stage nk-3 needed, stages nk-2 and nk-1 may be in flight
-    step(t + 1, W4 {}, F {}, T {}); // stage nk-2 needed, stage nk-1 may be in flight
-    step(t + 2, W0 {}, F {}, T {});
-    step(t + 3, W0 {}, F {}, F {});
+    if constexpr (NST % 2 != 0) // (the number of stages is even: an odd ring leaves one more step before the drain)
+    {
+        step(t, WM {}, T {}, T {});
+        t++;
+    }
+    // t == nk - NST (nk >= NST): everything has been requested; step nk-NST+i needs stage nk-NST+i+1 with NST-2-i younger stages
+    // behind it, the last step reads nothing
+    auto drain = [&](auto ic) __attribute__((always_inline))
+    {
+        constexpr int I = decltype(ic)::value;
+        if constexpr (I < NST - 1) step(t + I, std::integral_constant<int, vm_wait((NST - 2 - I) * NREQ)> {}, F {}, T {});
+    };
+    if constexpr (NST == 4)
+    {
+        step(t, std::integral_constant<int, vm_wait(2 * NREQ)> {}, F {}, T {});
+        step(t + 1, std::integral_constant<int, vm_wait(NREQ)> {}, F {}, T {});
+        step(t + 2, std::integral_constant<int, vm_wait(0)> {}, F {}, T {});
+        step(t + 3, std::integral_constant<int, vm_wait(0)> {}, F {}, F {});
+    }
+    else
+    {
+        drain(std::integral_constant<int, 0> {});
+        drain(std::integral_constant<int, 1> {});
+        drain(std::integral_constant<int, 2> {});
+        drain(std::integral_constant<int, 3> {});
+        drain(std::integral_constant<int, 4> {});
+        step(t + NST - 1, std::integral_constant<int, vm_wait(0)> {}, F {}, F {});
+    }
 #undef MMA
 #undef RA
 #undef RB
@@ -669,6 +723,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
                            g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
     const int       kg = elane >> 5;
+    const bool      finite = g.epi.finite != 0;
     // element offset of this elane's first value in block (0, 0): row em0 + ewm * WR + elane % 32, column en0 + ewn * 64 + 16 kg
     const long long lane_elem = c_off + (long long) (em0 + ewm * WR + (elane & 31)) * ldc + en0 + ewn * 64 + kg * 16;
     // block (i, j) -> the elane's 16 values after the power-of-two factors and relu
@@ -714,7 +769,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         constexpr int ESZ = decltype(esz_c)::value; // bytes per output element = 16-byte chunks per elane and block
         constexpr int RB = 64 * ESZ, CPR = RB / 16, NRD = RB / 32;
         // (PERSIST: behind the ring, which already holds the next tile; 1- and 2-byte outputs only, the host sees to that)
-        char*         stg = lds + (PERSIST && ESZ <= 2 ? FNST * STAGE : 0) + ewave * (32 * RB);
+        char*         stg = lds + (PERSIST && ESZ <= 2 ? NST * STAGE : 0) + ewave * (32 * RB);
         const int     row = elane & 31, swz = (row * CPR / 16) & (CPR - 1);
         constexpr bool RAW = decltype(raw_c)::value; // partial sums of a k-slice: no factors, no relu
         if constexpr (!PERSIST) __syncthreads(); // the slowest wavefront has taken its last fragments out of the ring
@@ -772,11 +827,15 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         // all 2^32 inputs); NaN, inf and values that round to inf (where clipping matters) are rare: the sum of |x| over
         // the elane's 16 values detects them and the block is then converted element by element
         walk(std::integral_constant<int, 2>(), [&](const float (&val)[16], uint32_t (&pk)[8]) __attribute__((always_inline)) {
-            float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            bool special = false;
+            if (!finite)
+            {
+                float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
-            const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
-            if (__builtin_amdgcn_ballot_w64(special) == 0)
+                for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
+                special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) < 0x1.ffp+127f);
+            }
+            if (finite || __builtin_amdgcn_ballot_w64(special) == 0)
             {
 #pragma unroll
                 for (int c = 0; c < 8; c++)
@@ -800,11 +859,15 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             walk(std::integral_constant<int, 1>(), [&](const float (&val)[16], uint32_t (&pk)[4]) __attribute__((always_inline)) {
                 // the hardware converter equals the reference's conversion on finite inputs; a block that holds inf or
                 // NaN (sum of magnitudes not finite) takes the exact converter
-                float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                bool special = false;
+                if (!finite)
+                {
+                    float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
-                const bool special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) <= 0x1.fffffep+127f);
-                if (__builtin_amdgcn_ballot_w64(special) == 0)
+                    for (int c = 0; c < 16; c++) sum[c & 3] += __builtin_fabsf(val[c]);
+                    special = !((sum[0] + sum[1]) + (sum[2] + sum[3]) <= 0x1.fffffep+127f);
+                }
+                if (finite || __builtin_amdgcn_ballot_w64(special) == 0)
                 {
 #pragma unroll
                     for (int c = 0; c < 4; c++) pk[c] = fp8_hw_pack4<MAN>(val[4 * c], val[4 * c + 1], val[4 * c + 2], val[4 * c + 3], cp.exp_bias, cp.clip_fp);
@@ -872,9 +935,9 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 
 // sets the dynamic-LDS limit once per kernel, then launches
 template<class K>
-hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s, int tile_m = FBM)
+hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s, int tile_m = FBM, int stages = FNST)
 {
-    const int lds_bytes = FNST * (tile_m * FBK + FBK * FBN);
+    const int lds_bytes = stages * (tile_m * FBK + FBK * FBN);
     if (!attr_done)
     {
         hipError_t e = hipFuncSetAttribute((const void*) kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);

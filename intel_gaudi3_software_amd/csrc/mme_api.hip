@@ -264,6 +264,9 @@ struct Fp8Plan
 {
     int fold_exp = 0;     // accumulators are multiplied by 2^fold_exp
     int scan_kind[2] = {-1, -1}; // -1: every code is exact in the hardware format; 0 / 1: mask kind to scan for
+    // mask kind whose absence also rules out inf and NaN among the operand's values (-1: the scan above already does, or the
+    // format has none): 0 any exponent-all-ones code, 1 only 0x7F / 0xFF
+    int nonfinite_kind[2] = {-1, -1};
 };
 
 Fp8Plan plan_fp8(const mme_hip_tensor* a, const mme_hip_tensor* b)
@@ -278,12 +281,14 @@ Fp8Plan plan_fp8(const mme_hip_tensor* a, const mme_hip_tensor* b)
             // full mode: exponent 15 is inf / NaN (finite 256..448 for the hardware); no-inf-nan mode: 0x7F is finite
             // (NaN for the hardware); minimal mode is the hardware's own format
             p.scan_kind[i] = t[i]->inf_nan_mode == 0 ? 0 : (t[i]->inf_nan_mode == 1 ? 1 : -1);
+            p.nonfinite_kind[i] = t[i]->inf_nan_mode == 2 ? 1 : -1; // minimal mode: 0x7F / 0xFF are NaN for Gaudi and hardware alike
         }
         else
         {
             p.fold_exp += 15 - (int) t[i]->fp_bias; // hardware e5m2 has bias 15
             // full mode is the hardware's own format; the other modes give finite meaning to exponent-31 codes
             p.scan_kind[i] = t[i]->inf_nan_mode == 0 ? -1 : 0;
+            p.nonfinite_kind[i] = t[i]->inf_nan_mode == 0 ? 0 : -1; // full mode: exponent 31 is inf / NaN for Gaudi and hardware alike
         }
     }
     return p;
@@ -526,6 +531,33 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     // alpha so far holds the caller's descale (or 1); fold the bias difference into the same multiplication
     if (int rc = fold_alpha(h, g.epi, fold)) return rc;
     const bool need_scan = (plan.scan_kind[0] >= 0 || plan.scan_kind[1] >= 0) && h->fp8_specials_policy == 0;
+    // Can a value that is not finite reach the output conversion?  Not when no operand holds an inf or NaN code (the caller's
+    // promise, or the checks below), the accumulators stay below 2^(log2 K + 26) in the hardware formats' units, and the only
+    // factor is the one power of two known here: the fast converters then skip their look-out for such values.
+    const bool in_kernel_check = need_scan && gemm_large_tile_checks_operands(g);
+    {
+        bool finite = h->fp8_specials_policy == MME_HIP_FP8_SPECIALS_ASSUME_NONE || in_kernel_check ||
+                      (plan.nonfinite_kind[0] < 0 && plan.nonfinite_kind[1] < 0 && need_scan);
+        uint32_t bits;
+        memcpy(&bits, &g.epi.alpha, 4);
+        const int ex = g.epi.has_alpha ? (int) ((bits >> 23) & 0xFF) - 127 : 0;
+        int       log2k = 0;
+        while ((1ll << log2k) < g.K) log2k++;
+        g.epi.finite = finite && !g.epi.col_exp && log2k + 26 + ex < 127;
+        const char* exp_env = getenv("MME_HIP_EXPERIMENT"); // (temporary: A/B switches for measurements)
+        const int          exp_mask = exp_env ? atoi(exp_env) : 0;
+        if (exp_mask & 1) g.epi.finite = 0;
+        // The plain large-tile fp8 kernel can hand that power of two to the matrix instruction (its block-scale operand) and
+        // save a multiplication per output.  Scaling before the fp32 accumulation equals scaling after it as long as nothing
+        // leaves the normal fp32 range either way: the smallest product is 2^-32 in the hardware formats' units (two e5m2
+        // denormals) and sums stay below 2^(log2 K + 26).
+        if (!(exp_mask & 2) && g.epi.has_alpha && !in_kernel_check && ex >= -94 && ex <= 100 && log2k + 26 + ex < 127 && log2k + 26 < 127 && gemm_large_tile_takes_mfma_scale(g))
+        {
+            g.epi.mfma_scale_exp = ex;
+            g.epi.alpha = 1.0f;
+            g.epi.has_alpha = 0;
+        }
+    }
     if (!need_scan)
     {
         HIP_TRY(h, launch_gemm(g, h->stream));
@@ -540,15 +572,18 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     g.skip_flag = flag;
     g.skip_epoch = epoch;
     g.skip_if = 1; // native variant: skipped when the scan found something
-    if (gemm_large_tile_checks_operands(g))
+    if (in_kernel_check)
     {
         g.chk = 1;
         const mme_hip_tensor* t[2] = {ta, tb};
         uint32_t              mask[2], add[2];
         for (int i = 0; i < 2; i++)
         {
-            // a byte b is special when (b & m) == m: m = the exponent field (kind 0) or all of 0x7F (kind 1: only 0x7F / 0xFF)
-            const uint32_t m = plan.scan_kind[i] < 0 ? 0u : (plan.scan_kind[i] == 1 ? 0x7Fu : (t[i]->dtype == MME_HIP_FP8_143 ? 0x78u : 0x7Cu));
+            // a byte b is special when (b & m) == m: m = the exponent field (kind 0) or all of 0x7F (kind 1: only 0x7F / 0xFF).
+            // An operand in its hardware-native mode is looked at as well, for its inf / NaN codes: the exact fall-back
+            // converts those values like any other, and the native kernel's epilogue may count on finite accumulators.
+            const int      kind = plan.scan_kind[i] >= 0 ? plan.scan_kind[i] : plan.nonfinite_kind[i];
+            const uint32_t m = kind < 0 ? 0u : (kind == 1 ? 0x7Fu : (t[i]->dtype == MME_HIP_FP8_143 ? 0x78u : 0x7Cu));
             mask[i] = m * 0x01010101u;
             add[i] = m ? (0x80u - m) * 0x01010101u : 0u;
         }
@@ -578,10 +613,12 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     {
         uint32_t bits;
         memcpy(&bits, &g.epi.alpha, 4);
-        int e = g.epi.has_alpha ? (int) ((bits >> 23) & 0xFF) - 127 : 0;
+        int e = (g.epi.has_alpha ? (int) ((bits >> 23) & 0xFF) - 127 : 0) + g.epi.mfma_scale_exp;
         e -= fold; // decoded operands carry their true values
         g2.epi.alpha = pow2f(e);
         g2.epi.has_alpha = e != 0;
+        g2.epi.mfma_scale_exp = 0;
+        g2.epi.finite = 0; // (the decoded operands may hold inf and NaN)
     }
     g2.skip_if = 0; // decoded variant: skipped unless the scan found something
     g2.split_k = g.split_k;

@@ -106,6 +106,13 @@ struct GemmEpilogue
     int            has_alpha;
     const int32_t* col_exp;         // per f_b power-of-two exponents or NULL
     int            fast_cast;
+    // the host can rule out NaN, infinite and overflowing values before the cast (operands without such codes, a bounded
+    // reduction, one known power-of-two factor): the fast converters then need not look for them
+    int            finite;
+    // fp8 large-tile kernels: power-of-two exponent handed to the matrix instruction's block-scale operand instead of a
+    // multiplication per output (the host folds alpha into it when no product or sum can leave the fp32 range either way;
+    // has_alpha is then 0)
+    int            mfma_scale_exp;
 };
 
 struct GemmProblem
@@ -144,6 +151,8 @@ int        gemm_fast_pick_split_k(const GemmProblem& p, int num_cus); // 0: the 
 hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s);
 // the kernel this problem takes can check its fp8 operands for special codes itself (GemmProblem::chk)
 bool       gemm_large_tile_checks_operands(const GemmProblem& p);
+// the kernel this problem takes applies GemmEpilogue::mfma_scale_exp (the plain fp8 kernel with one workgroup per 256 x 256 tile)
+bool       gemm_large_tile_takes_mfma_scale(const GemmProblem& p);
 
 // forward convolution fast path (conv_fwd_fast.hip): bf16, 3x3, 64 -> 64 channels, stride 1, padding 1, dense NHWC
 bool       conv_fwd_fast_applicable(int dtype, int C, int K, int S, int R, int Q, int W, int H, int D, const int stride[4], const int dil[4],
