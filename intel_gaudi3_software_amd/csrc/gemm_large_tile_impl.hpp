@@ -177,8 +177,9 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // CHK (fp8, AMODE 0, whole 256-row tiles): the kernel inspects the operand bytes on their way to the matrix cores for codes
 // that the hardware's fp8 formats read differently from Gaudi's (GemmProblem::chk_*) and raises the problem's flag when it
 // meets one.  Every 64-byte stage of an operand row is looked at by exactly one of the workgroups that read it (stage t of
-// the A rows by the tile column t mod tiles_n, of the B columns by the tile row t mod tiles_m), a few vector instructions
-// in the shadow of the matrix instructions, so a clean operand costs no extra pass over memory and no extra launch.
+// the A rows by the tile column t mod tiles_n, of the B columns by the tile row t mod tiles_m): when its turn comes, each
+// wavefront reads an eighth of that part of the stage once more from LDS and tests the bytes, a few vector instructions in
+// the shadow of the matrix instructions, so a clean operand costs no extra pass over memory and no extra launch.
 // NST: stages of the ring (default 4).  What a compute unit can draw from L2 / memory is the bytes it has in flight divided
 // by the latency, so a kernel whose stages are small (the 128-row tile: 24 KiB) keeps more of them in flight: six stages,
 // 144 KiB.  The reduction then has to be at least NST stages long.
@@ -561,19 +562,19 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     if (LOADS) issue_a(u, t + NST, slot);
 #define LB(u) \
     if (LOADS) issue_b(u, t + NST, slot);
-#define CA(i) \
-    if (CHK && do_a && wn == i) chk_frag(f.a[i], chk_ma, chk_aa);
-#define CB(j) \
-    if (CHK && do_b && wm == j) chk_frag(f.b[j], chk_mb, chk_ab);
-    auto chk_frag = [&](const v8i& fr, uint32_t mask, uint32_t add) __attribute__((always_inline))
+    // the look itself: this wavefront's eighth (2 KiB) of one operand's part of a stage, straight from LDS (the swizzled
+    // placement does not matter, every byte of the part is an operand byte)
+    auto chk_scan = [&](const char* part, uint32_t mask, uint32_t add) __attribute__((always_inline))
     {
-#pragma unroll
-        for (int q = 0; q < 8; q += 2) chk_bad |= (((uint32_t) fr[q] & mask) + add) | (((uint32_t) fr[q + 1] & mask) + add);
+        const v4i x0 = *(const v4i*) (part + wave * 2048 + lane * 16), x1 = *(const v4i*) (part + wave * 2048 + 1024 + lane * 16);
+        chk_bad |= (((uint32_t) x0.x & mask) + add) | (((uint32_t) x0.y & mask) + add);
+        chk_bad |= (((uint32_t) x0.z & mask) + add) | (((uint32_t) x0.w & mask) + add);
+        chk_bad |= (((uint32_t) x1.x & mask) + add) | (((uint32_t) x1.y & mask) + add);
+        chk_bad |= (((uint32_t) x1.z & mask) + add) | (((uint32_t) x1.w & mask) + add);
     };
-    // stages until this workgroup's next turn to look at the A rows / B columns of its tile.  The four wavefronts with the same
-    // wm hold the same four A fragments and take one each (fragment i by the wavefront with wn == i); the two wavefronts with
-    // the same wn hold the same two B fragments and take one each: the work of a turn is spread evenly over the SIMDs
-    int chk_ca = cur_tn, chk_cb = cur_tm;
+    // steps until this workgroup's next turn to look at the A part / B part of a stage: stage s of the A rows falls to the tile
+    // column s mod tiles_n, of the B columns to the tile row s mod tiles_m; step t looks at stage t + 1 (stage 0 right here)
+    int chk_ca = (cur_tn + tiles_n - 1) % tiles_n, chk_cb = (cur_tm + tiles_m - 1) % tiles_m;
     // the constants of the check, read from the kernel arguments once and pinned in scalar registers: a read inside a step
     // would wait on the counter that the step's LDS reads share
     uint32_t chk_ma = 0, chk_aa = 0, chk_mb = 0, chk_ab = 0;
@@ -584,6 +585,8 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         asm volatile("" : "+s"(chk_ma), "+s"(chk_aa), "+s"(chk_mb), "+s"(chk_ab));
         chk_a_mine = chk_ma != 0;
         chk_b_mine = chk_mb != 0;
+        if (cur_tn == 0 && chk_a_mine) chk_scan(lds, chk_ma, chk_aa);
+        if (cur_tm == 0 && chk_b_mine) chk_scan(lds + A_BYTES, chk_mb, chk_ab);
     }
     // One stage: 8 MFMAs; after the first one wait until stage t+1 has landed in every wavefront's view (WAITC leaves the
     // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
@@ -596,32 +599,36 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         constexpr bool RN = decltype(readnext)::value;
         const char*    st = lds + ((t + 1) % NST) * STAGE;
         const int      slot = t % NST;
-        bool           do_a = false, do_b = false;
-        if constexpr (CHK)
-        {
-            do_a = chk_ca == 0 && chk_a_mine;
-            do_b = chk_cb == 0 && chk_b_mine;
-            chk_ca = chk_ca == 0 ? tiles_n - 1 : chk_ca - 1;
-            chk_cb = chk_cb == 0 ? tiles_m - 1 : chk_cb - 1;
-        }
         MMA(0, 0);
         FENCE;
         if (RN)
         {
             __builtin_amdgcn_s_waitcnt(WAITC);
             __builtin_amdgcn_s_barrier();
+            if constexpr (CHK)
+            {
+                // stage t + 1 has landed: one branch per step, the look is a cold block that touches no fragment register
+                const bool do_a = chk_ca == 0 && chk_a_mine, do_b = chk_cb == 0 && chk_b_mine;
+                chk_ca = chk_ca == 0 ? tiles_n - 1 : chk_ca - 1;
+                chk_cb = chk_cb == 0 ? tiles_m - 1 : chk_cb - 1;
+                if (__builtin_expect(do_a || do_b, 0))
+                {
+                    if (do_a) chk_scan(st, chk_ma, chk_aa);
+                    if (do_b) chk_scan(st + A_BYTES, chk_mb, chk_ab);
+                }
+            }
         }
         FENCE;
         MMA(0, 1); FENCE;
         if constexpr (NI == 4)
         {
-            CA(0) RA(0) LA(0) MMA(1, 0); FENCE;
+            RA(0) LA(0) MMA(1, 0); FENCE;
             MMA(1, 1); FENCE;
-            CA(1) RA(1) LA(1) MMA(2, 0); FENCE;
+            RA(1) LA(1) MMA(2, 0); FENCE;
             MMA(2, 1); FENCE;
-            CA(2) RA(2) LB(0) MMA(3, 0); FENCE;
-            CB(0) RB(0) LB(1) MMA(3, 1); FENCE;
-            CA(3) CB(1) RA(3) RB(1) FENCE;
+            RA(2) LB(0) MMA(3, 0); FENCE;
+            RB(0) LB(1) MMA(3, 1); FENCE;
+            RA(3) RB(1) FENCE;
         }
         else
         {
@@ -675,8 +682,6 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 #undef RB
 #undef LA
 #undef LB
-#undef CA
-#undef CB
     if constexpr (CHK)
     {
         if (chk_bad & 0x80808080u) *const_cast<uint32_t*>((const uint32_t*) g.skip_flag) = g.skip_epoch;

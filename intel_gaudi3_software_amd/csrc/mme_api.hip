@@ -544,14 +544,12 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         int       log2k = 0;
         while ((1ll << log2k) < g.K) log2k++;
         g.epi.finite = finite && !g.epi.col_exp && log2k + 26 + ex < 127;
-        const char* exp_env = getenv("MME_HIP_EXPERIMENT"); // (temporary: A/B switches for measurements)
-        const int          exp_mask = exp_env ? atoi(exp_env) : 0;
-        if (exp_mask & 1) g.epi.finite = 0;
+
         // The plain large-tile fp8 kernel can hand that power of two to the matrix instruction (its block-scale operand) and
         // save a multiplication per output.  Scaling before the fp32 accumulation equals scaling after it as long as nothing
         // leaves the normal fp32 range either way: the smallest product is 2^-32 in the hardware formats' units (two e5m2
         // denormals) and sums stay below 2^(log2 K + 26).
-        if (!(exp_mask & 2) && g.epi.has_alpha && !in_kernel_check && ex >= -94 && ex <= 100 && log2k + 26 + ex < 127 && log2k + 26 < 127 && gemm_large_tile_takes_mfma_scale(g))
+        if (g.epi.has_alpha && !in_kernel_check && ex >= -94 && ex <= 100 && log2k + 26 + ex < 127 && log2k + 26 < 127 && gemm_large_tile_takes_mfma_scale(g))
         {
             g.epi.mfma_scale_exp = ex;
             g.epi.alpha = 1.0f;
@@ -588,6 +586,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
             add[i] = m ? (0x80u - m) * 0x01010101u : 0u;
         }
         g.chk_mask_a = mask[0], g.chk_add_a = add[0], g.chk_mask_b = mask[1], g.chk_add_b = add[1];
+
     }
     else
         HIP_TRY(h, launch_fp8_special_scan2(flag, epoch, a_base, span_elements(ta), ta->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[0], b_base,
