@@ -86,6 +86,37 @@ class Bench:
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / n * 1e-3
 
+    def clocked(self, fn, n=30):
+        """The shader clock the large-tile kernels ran at during n back-to-back calls of fn, and how long a workgroup took
+        (stamps taken inside the kernels; the published peak rates are quoted at 2400 MHz)."""
+        self.calc.clockProbe(True)
+        self.calc.readClockProbe()
+        for _ in range(n):
+            fn()
+        r = self.calc.readClockProbe()
+        self.calc.clockProbe(False)
+        return {"shader_clock_mhz": round(r["shader_mhz"]), "workgroup_us_mean": round(r["workgroup_us_mean"], 2),
+                "workgroup_us_max": round(r["workgroup_us_max"], 2), "workgroups_seen": r["workgroups"]}
+
+    def matrix_core_ceiling(self, dtype):
+        """What back-to-back matrix instructions with operands in registers sustain on this device: with all-zero operands
+        (the published rate) and with operands that change from instruction to instruction (power management lowers the clock)."""
+        out = {}
+        for name, rnd in (("zero_operands", 0), ("random_operands", 1)):
+            tf, mhz = self.calc.matrixCoreRate(dtype, rnd, iters=4096, launches=10)
+            out[name] = {"TFLOP/s": round(tf, 1), "shader_clock_mhz": round(mhz)}
+        return out
+
+    def pmc_calibration(self):
+        """Five launches of a plain copy of 2^26 floats (256 MiB read, 256 MiB written): the unit of FETCH_SIZE / WRITE_SIZE."""
+        torch = self.torch
+        with torch.cuda.stream(self.stream):
+            src = torch.ones(1 << 26, dtype=torch.float32, device="cuda")
+            dst = torch.empty_like(src)
+            for _ in range(5):
+                torch.add(src, 0.0, out=dst)
+        torch.cuda.synchronize()
+
     def checker(self):
         """(library, kind, prefix): the compiled reference where it has been built, else the oracle restatement."""
         import oracle
@@ -171,15 +202,6 @@ def run_c2(b):
     def step():
         calc.doBatchGemm(Y, X, W, abi.OP_AB, epilogue=epi)
 
-    if args.pmc_calibration:
-        with torch.cuda.stream(b.stream):
-            src = torch.ones(1 << 26, dtype=torch.float32, device="cuda")
-            dst = torch.empty_like(src)
-            for _ in range(5):
-                torch.add(src, 0.0, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
-
     # The library's default policy (MME_HIP_FP8_SPECIALS_CHECK) looks for exponent-all-ones codes, which mean inf / NaN to
     # Gaudi and numbers to the matrix cores, while the kernel multiplies, and enqueues the exact fall-back behind it; a
     # caller whose operands come out of a saturating quantiser, as here, may promise that there are none
@@ -222,6 +244,16 @@ def run_c2(b):
                                      "kernel": "gemm_fp8_fast_kernel<0, false>",
                                      "policy": "the caller promises operands without exponent-all-ones codes (they come out of the saturating quantiser)"}},
     }
+
+    # the clock the kernel ran at (all-zero operands would let the device hold 2400 MHz; these operands do not), and what
+    # bare matrix instructions sustain on zero and on random operands
+    result["roofline"]["clock"] = b.clocked(step, n=50)
+    calc.setFp8SpecialsPolicy(abi.FP8_SPECIALS_ASSUME_NONE)
+    result["roofline"]["assume_none"]["clock"] = b.clocked(step, n=50)
+    calc.setFp8SpecialsPolicy(abi.FP8_SPECIALS_CHECK)
+    result["roofline"]["matrix_core_ceiling"] = b.matrix_core_ceiling(abi.FP8_143)
+    step()  # (the parity check below reads the output of a default-policy call)
+    torch.cuda.synchronize()
 
     # ---- parity of the timed output on M-slabs + CPU baseline --------------------------------------------------------
     if b.cpu:
@@ -273,6 +305,7 @@ def run_c1(b):
     flop = 2.0 * n ** 3
     res = {"workload": "bf16 GEMM 512^3 -> fp32 (configs[0])", "value": round(flop / t / 1e12, 2), "unit": "TFLOP/s",
            "roofline": mfma_roofline(flop, t, "bf16", "gemm_2byte_fast128_kernel")}
+    res["roofline"]["clock"] = b.clocked(lambda: calc.doBatchGemm(Y1, A1, B1, abi.OP_AB))
     if b.cpu:
         want = np.zeros(n * n, np.float32)
         da, dw, do = abi.make_tensor(a.ctypes.data, [n, n], abi.BF16), abi.make_tensor(w.ctypes.data, [n, n], abi.BF16), abi.make_tensor(want.ctypes.data, [n, n], abi.FP32)
@@ -356,6 +389,9 @@ def _run_c4(b, op):
     kernel = "conv_2byte_fast128_kernel" if op == abi.OP_DEDX else "conv_dedw_2byte_fast128_kernel + splitk_reduce_kernel"
     res = {"workload": "bf16 conv2d %s N=32 28x28 C=K=256 3x3 s1 p1, fp32 output (configs[3])" % name, "value": round(flop / t / 1e12, 2),
            "unit": "TFLOP/s", "roofline": mfma_roofline(flop, t, "bf16", kernel)}
+    res["roofline"]["clock"] = b.clocked(lambda: calc.doConvolution(OT, XT, WT, YT, cp, op))
+    if op == abi.OP_DEDX:
+        res["roofline"]["matrix_core_ceiling"] = b.matrix_core_ceiling(abi.BF16)
     if b.cpu:
         want = np.zeros(int(np.prod(osz)), np.float32)
         p = abi.make_conv_params(2, (1, 1, 0), (1, 1, 1), (1, 1, 1))
@@ -420,6 +456,7 @@ def run_c5(b):
                        "scales, fp8_143 output (configs[4]); library default policy for fp8 special codes", "value": round(flop / t / 1e12, 2),
            "unit": "TFLOP/s", "roofline": mfma_roofline(flop, t, "fp8", "gemm_fp8_persistent_chk_kernel<2, false>"),
            "scale_exp": {"a": sa, "out": so, "b_per_channel_min_max": [int(sb.min()), int(sb.max())]}}
+    res["roofline"]["clock"] = b.clocked(lambda: calc.doBatchGemm(Y5, A5, B5, abi.OP_AB, epilogue=e5), n=10)
     if b.cpu:
         orc = b.oracle_lib()
         r = 64
@@ -532,6 +569,8 @@ def main():
         sys.exit(2)
 
     b = Bench(args)
+    if args.pmc_calibration:
+        b.pmc_calibration()
     if args.only and args.only != "c2":
         if args.only not in WORKLOADS:
             print("unknown workload %r" % args.only, file=sys.stderr)

@@ -225,6 +225,26 @@ int mme_hip_synchronize(mme_hip_handle h);
 int mme_hip_set_wait_limit(mme_hip_handle h, unsigned polls);
 
 /*
+ * Diagnostics, no counterpart in the reference.  The device lowers its shader clock under load, and by how much depends on
+ * the operand values (all-zero operands toggle nothing), so a kernel's distance from the published peak rate says little
+ * without the clock it ran at.
+ *
+ * mme_hip_clock_probe(h, 1): from now on every workgroup of the large-tile contraction kernels notes the shader clock
+ * counter and the constant 100 MHz counter when it starts and when it ends (up to 4096 workgroups per launch, 128 KiB of
+ * device memory, allocated here); (h, 0) switches that off again.  mme_hip_clock_probe_read synchronises the stream and
+ * reports, over the workgroups that ran since the last read: the clock (shader clocks per 100 MHz tick x 100), the mean and
+ * the longest time a workgroup took, and their number.
+ *
+ * mme_hip_matrix_core_rate: `launches` launches of a loop of `iters` x 8 matrix instructions per wavefront (32x32x64 fp8
+ * for MME_HIP_FP8_143, 32x32x16 for MME_HIP_BF16) on every compute unit, operands in registers, all zero or
+ * (random_operands != 0) random and changing from instruction to instruction: the rate the matrix cores sustain on this
+ * device with nothing else to do, and the clock they held.
+ */
+int mme_hip_clock_probe(mme_hip_handle h, int enable);
+int mme_hip_clock_probe_read(mme_hip_handle h, double* shader_mhz, double* mean_us, double* max_us, int* workgroups);
+int mme_hip_matrix_core_rate(mme_hip_handle h, int dtype, int random_operands, int iters, int launches, double* tflops, double* shader_mhz);
+
+/*
  * clipFp / clipFpInfIn of the operand conversion, for the device-pointer contraction entry points (the host-pointer
  * ones take them per call).  On Gaudi3 only the tf32 flavour reads them: its operands are rounded from fp32 to tf32 on
  * entry and an overflow to infinity is clipped to the largest finite value when clip_fp is set (and, for an infinite

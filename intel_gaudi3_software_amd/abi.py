@@ -137,6 +137,9 @@ def load_library():
     L.mme_hip_set_stream.argtypes = [vp, vp]
     L.mme_hip_synchronize.argtypes = [vp]
     L.mme_hip_set_wait_limit.argtypes = [vp, C.c_uint]
+    L.mme_hip_clock_probe.argtypes = [vp, C.c_int]
+    L.mme_hip_clock_probe_read.argtypes = [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int)]
+    L.mme_hip_matrix_core_rate.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.mme_hip_set_fp8_specials_policy.argtypes = [vp, C.c_int]
     L.mme_hip_set_operand_clip.argtypes = [vp, C.c_int, C.c_int]
     L.mme_hip_batch_gemm.argtypes = [vp, _TP, _TP, _TP, C.c_int, C.c_int, C.c_int, C.c_int]

@@ -248,6 +248,27 @@ class HipCalculator:
         next synchronize()."""
         self._check(self._lib.mme_hip_set_wait_limit(self._h, polls))
 
+    def clockProbe(self, enable=True):
+        """Diagnostics (mme_hip_clock_probe): the large-tile kernels note clock counters per workgroup while this is on."""
+        self._check(self._lib.mme_hip_clock_probe(self._h, int(bool(enable))))
+
+    def readClockProbe(self):
+        """Synchronises and returns {shader_mhz, workgroup_us_mean, workgroup_us_max, workgroups} over the workgroups that ran
+        since the last read (mme_hip_clock_probe_read)."""
+        import ctypes as C
+        mhz, mean, worst, n = C.c_double(), C.c_double(), C.c_double(), C.c_int()
+        self._check(self._lib.mme_hip_clock_probe_read(self._h, C.byref(mhz), C.byref(mean), C.byref(worst), C.byref(n)))
+        self._in_flight.clear()
+        return {"shader_mhz": mhz.value, "workgroup_us_mean": mean.value, "workgroup_us_max": worst.value, "workgroups": n.value}
+
+    def matrixCoreRate(self, dtype, random_operands, iters=4096, launches=10):
+        """(TFLOP/s, shader clock in MHz) of back-to-back matrix instructions with operands in registers
+        (mme_hip_matrix_core_rate): what the matrix cores sustain on this device and this kind of data."""
+        import ctypes as C
+        tf, mhz = C.c_double(), C.c_double()
+        self._check(self._lib.mme_hip_matrix_core_rate(self._h, dtype, int(bool(random_operands)), iters, launches, C.byref(tf), C.byref(mhz)))
+        return tf.value, mhz.value
+
     def setFp8SpecialsPolicy(self, policy):
         self._check(self._lib.mme_hip_set_fp8_specials_policy(self._h, policy))
 

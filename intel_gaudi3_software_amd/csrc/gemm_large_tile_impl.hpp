@@ -183,9 +183,16 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // NST: stages of the ring (default 4).  What a compute unit can draw from L2 / memory is the bytes it has in flight divided
 // by the latency, so a kernel whose stages are small (the 128-row tile: 24 KiB) keeps more of them in flight: six stages,
 // 144 KiB.  The reduction then has to be at least NST stages long.
+__device__ __forceinline__ void clock_probe_stamp(KARG GemmProblem& g, int at_end);
+#ifdef MME_X_FROM
+#define PHASE(k) do { if (g.clock_probe) { if (MME_X_FROM == (k)) clock_probe_stamp(g, 0); if (MME_X_TO == (k)) clock_probe_stamp(g, 1); } } while (0)
+#else
+#define PHASE(k) do { } while (0)
+#endif
 template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST>
-__device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
+__device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 {
+    PHASE(0);
     static_assert(NST >= 4 && NST <= 6 && (!PERSIST || NST == FNST), "ring depth");
     static_assert(!CHK || (ES == 1 && AMODE == 0 && TM == FBM && !RG), "operand checks: fp8, plain k-contiguous A, whole 256-row tiles");
     static_assert(!PERSIST || (AMODE == 0 && TM == FBM && !RG), "the persistent schedule: plain k-contiguous A, whole 256-row tiles");
@@ -365,7 +372,32 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 off0 += (long long) (g.A.gather_y ? pp.c[d] + g.A.pad[d] : pp.c[d] * g.A.cstride[d] - g.A.pad[d]) * g.A.src_stride[d];
             ga[u] = A + off0 * ES + c * 16;
             if (m0 + r < g.M)
-                for (int t = 0; t < ntaps; t++) tap_ok[u] |= (conv_offset(g.A, pp, t) >= 0 ? 1u : 0u) << t;
+            {
+                // which taps land inside the tensor: range checks per dimension, the taps counted up as (s, r, q) digits
+                // (no division: the gather form of col2im comes here with unit strides only)
+                int ts[3] = {0, 0, 0};
+                for (int t = 0; t < ntaps; t++)
+                {
+                    bool ok = true;
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                    {
+                        const int td = d < 3 ? ts[d] * g.A.dil[d] : 0;
+                        const int pos = g.A.gather_y ? pp.c[d] + g.A.pad[d] - td : pp.c[d] * g.A.cstride[d] + td - g.A.pad[d];
+                        ok = ok && pos >= 0 && pos < g.A.src[d];
+                    }
+                    tap_ok[u] |= (ok ? 1u : 0u) << t;
+                    if (++ts[0] == g.A.ktap[0])
+                    {
+                        ts[0] = 0;
+                        if (++ts[1] == g.A.ktap[1])
+                        {
+                            ts[1] = 0;
+                            ts[2]++;
+                        }
+                    }
+                }
+            }
         }
         if (g.B.kind == VIEW_TAPPED)
 #pragma unroll
@@ -410,6 +442,17 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             for (int d = 0; d < 4; d++) w_pc[u][d] = pp.c[d];
         }
     }
+    // the address of the zero page, fetched once and pinned in two scalar registers: left to itself the compiler re-reads it
+    // from the global offset table in every step, and the wait for that scalar load also waits for the step's LDS reads
+    uint32_t zero_lo = 0, zero_hi = 0;
+    if constexpr (AMODE == 3 || GATHER)
+    {
+        const uint64_t z = (uint64_t) (uintptr_t) gf_zero_page;
+        zero_lo = (uint32_t) z;
+        zero_hi = (uint32_t) (z >> 32);
+        asm volatile("" : "+s"(zero_lo), "+s"(zero_hi));
+    }
+    auto zero_page = [&]() __attribute__((always_inline)) { return (const uint8_t*) (uintptr_t) (((uint64_t) zero_hi << 32) | zero_lo); };
     auto issue_a = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
         if constexpr (AMODE == 3)
@@ -424,7 +467,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 ok = ok && pos >= 0 && pos < g.A.src[d];
                 off += (long long) pos * g.A.src_stride[d] * ES;
             }
-            const uint8_t* src = ok ? A + off : (const uint8_t*) gf_zero_page;
+            const uint8_t* src = ok ? A + off : zero_page();
             dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
             // next stage: 32 (2-byte elements) or 64 (fp8) pixels further
             int carry = FBK / ES;
@@ -446,7 +489,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         else if constexpr (GATHER)
         {
             const bool     ok = (tap_ok[u] >> g_tap) & 1u;
-            const uint8_t* src = ok ? ga[u] + g_delta_a : (const uint8_t*) gf_zero_page;
+            const uint8_t* src = ok ? ga[u] + g_delta_a : zero_page();
             dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
         }
         else
@@ -486,6 +529,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             }
         }
     };
+    PHASE(1);
     issue_prologue();
     for (int walk_it = 0;;) // (one pass unless PERSIST)
     {
@@ -503,6 +547,7 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
                 for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
     }
     __syncthreads();
+    PHASE(2);
     auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
     {
         if constexpr (A_KC) read_a(fr, i, st, wm * WR, lane);
@@ -511,15 +556,22 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         else
             read_a_tr16<TM>(fr, i, st, wm, lane);
     };
-    Frags f;
+    // The 128-row tile (two A fragments per wavefront) has registers to spare and only four matrix steps per stage to hide
+    // an LDS read behind: it keeps two fragment sets and fills the one for stage t+1 in one go at the start of step t, so no
+    // matrix instruction of a step waits for LDS.  The 256-row tile refills its single set register by register.
+#ifndef MME_X_DBUF
+#define MME_X_DBUF 1
+#endif
+    constexpr bool DBUF = NI == 2 && MME_X_DBUF;
+    Frags fr[DBUF ? 2 : 1];
 #pragma unroll
-    for (int i = 0; i < NI; i++) read_a_any(f, i, lds);
+    for (int i = 0; i < NI; i++) read_a_any(fr[0], i, lds);
 #pragma unroll
-    for (int j = 0; j < 2; j++) read_b(f, j, lds);
+    for (int j = 0; j < 2; j++) read_b(fr[0], j, lds);
 
     constexpr bool MSCALE = ES == 1 && AMODE == 0 && TM == FBM && !RG && !PERSIST && !CHK;
     const int      mfma_scale_a = 127 + (MSCALE ? g.epi.mfma_scale_exp : 0);
-    auto mma = [&](int i, int j) __attribute__((always_inline))
+    auto mma = [&](Frags & f, int i, int j) __attribute__((always_inline))
     {
         if constexpr (ES == 1)
         {
@@ -553,15 +605,24 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
             }
         }
     };
-#define MMA(i, j) mma(i, j)
+#ifndef MME_X_NOMMA
+#define MME_X_NOMMA 0
+#endif
+#ifndef MME_X_NOREAD
+#define MME_X_NOREAD 0
+#endif
+#ifndef MME_X_NODMA
+#define MME_X_NODMA 0
+#endif
+#define MMA(i, j) if (!MME_X_NOMMA) mma(fc, i, j)
 #define RA(i) \
-    if (RN) read_a_any(f, i, st);
+    if (RN && !MME_X_NOREAD) read_a_any(fn, i, st);
 #define RB(j) \
-    if (RN) read_b(f, j, st);
+    if (RN && !MME_X_NOREAD) read_b(fn, j, st);
 #define LA(u) \
-    if (LOADS) issue_a(u, t + NST, slot);
+    if (LOADS && !MME_X_NODMA) issue_a(u, t + NST, slot);
 #define LB(u) \
-    if (LOADS) issue_b(u, t + NST, slot);
+    if (LOADS && !MME_X_NODMA) issue_b(u, t + NST, slot);
     // the look itself: this wavefront's eighth (2 KiB) of one operand's part of a stage, straight from LDS (the swizzled
     // placement does not matter, every byte of the part is an operand byte)
     auto chk_scan = [&](const char* part, uint32_t mask, uint32_t add) __attribute__((always_inline))
@@ -592,11 +653,14 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
     // other wavefront on the SIMD covers the tail of that latency); request stage t+4 into the slot of stage t, whose
     // fragments every wavefront read during the previous step (the barrier above orders those reads before this request).
-    auto step = [&](int t, auto waitc, auto loads, auto readnext) __attribute__((always_inline))
+    auto step = [&](int t, auto waitc, auto loads, auto readnext, auto parity) __attribute__((always_inline))
     {
         constexpr int  WAITC = decltype(waitc)::value;
         constexpr bool LOADS = decltype(loads)::value;
         constexpr bool RN = decltype(readnext)::value;
+        constexpr int  PAR = decltype(parity)::value; // t mod 2: which fragment set holds stage t (DBUF)
+        Frags&         fc = fr[DBUF ? PAR : 0];
+        Frags&         fn = fr[DBUF ? 1 - PAR : 0];
         const char*    st = lds + ((t + 1) % NST) * STAGE;
         const int      slot = t % NST;
         MMA(0, 0);
@@ -632,10 +696,11 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         }
         else
         {
-            // 128-row tile: four MFMAs per stage, three requests
-            RA(0) LA(0) MMA(1, 0); FENCE;
-            RB(0) LB(0) MMA(1, 1); FENCE;
-            RA(1) RB(1) LB(1) FENCE;
+            // 128-row tile: four matrix steps per stage, three requests; all of stage t+1 goes to the other fragment set now
+            RA(0) RB(0) RA(1) RB(1) FENCE;
+            LA(0) LB(0) LB(1) FENCE;
+            MMA(1, 0); FENCE;
+            MMA(1, 1); FENCE;
         }
     };
     // at the wait of step t the stages t+1 .. t+NST-1 have been requested; stage t+1 is needed, so the younger NST-2 stages of
@@ -643,30 +708,34 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     using WM = std::integral_constant<int, vm_wait((NST - 2) * NREQ)>;
     using T = std::true_type;
     using F = std::false_type;
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
     int t = 0;
     for (; t + NST + 1 < nk; t += 2) // steps 0 .. nk-NST-1 request stages NST .. nk-1
     {
-        step(t, WM {}, T {}, T {});
-        step(t + 1, WM {}, T {}, T {});
+        step(t, WM {}, T {}, T {}, P0 {});
+        step(t + 1, WM {}, T {}, T {}, P1 {});
     }
     if constexpr (NST % 2 != 0) // (the number of stages is even: an odd ring leaves one more step before the drain)
     {
-        step(t, WM {}, T {}, T {});
+        step(t, WM {}, T {}, T {}, P0 {});
         t++;
     }
+    constexpr int DP = NST % 2; // parity of the first step of the drain
     // t == nk - NST (nk >= NST): everything has been requested; step nk-NST+i needs stage nk-NST+i+1 with NST-2-i younger stages
     // behind it, the last step reads nothing
     auto drain = [&](auto ic) __attribute__((always_inline))
     {
         constexpr int I = decltype(ic)::value;
-        if constexpr (I < NST - 1) step(t + I, std::integral_constant<int, vm_wait((NST - 2 - I) * NREQ)> {}, F {}, T {});
+        if constexpr (I < NST - 1)
+            step(t + I, std::integral_constant<int, vm_wait((NST - 2 - I) * NREQ)> {}, F {}, T {}, std::integral_constant<int, (DP + I) % 2> {});
     };
     if constexpr (NST == 4)
     {
-        step(t, std::integral_constant<int, vm_wait(2 * NREQ)> {}, F {}, T {});
-        step(t + 1, std::integral_constant<int, vm_wait(NREQ)> {}, F {}, T {});
-        step(t + 2, std::integral_constant<int, vm_wait(0)> {}, F {}, T {});
-        step(t + 3, std::integral_constant<int, vm_wait(0)> {}, F {}, F {});
+        step(t, std::integral_constant<int, vm_wait(2 * NREQ)> {}, F {}, T {}, P0 {});
+        step(t + 1, std::integral_constant<int, vm_wait(NREQ)> {}, F {}, T {}, P1 {});
+        step(t + 2, std::integral_constant<int, vm_wait(0)> {}, F {}, T {}, P0 {});
+        step(t + 3, std::integral_constant<int, vm_wait(0)> {}, F {}, F {}, P1 {});
     }
     else
     {
@@ -675,8 +744,9 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
         drain(std::integral_constant<int, 2> {});
         drain(std::integral_constant<int, 3> {});
         drain(std::integral_constant<int, 4> {});
-        step(t + NST - 1, std::integral_constant<int, vm_wait(0)> {}, F {}, F {});
+        step(t + NST - 1, std::integral_constant<int, vm_wait(0)> {}, F {}, F {}, std::integral_constant<int, (DP + NST - 1) % 2> {});
     }
+    PHASE(3);
 #undef MMA
 #undef RA
 #undef RB
@@ -935,6 +1005,35 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
     (void) esz;
     if (!PERSIST || !has_next) break;
     } // walk over tiles
+}
+
+// GemmProblem::clock_probe (diagnostics, normally NULL): the first lane of a workgroup notes the shader clock counter and
+// the constant 100 MHz counter when the workgroup starts (cells 0, 1 of its four) and when its first wavefront ends (2, 3);
+// the host derives the clock the kernel really ran at and the time a workgroup took from them.
+__device__ __forceinline__ void clock_probe_stamp(KARG GemmProblem& g, int at_end)
+{
+    uint64_t* probe = g.clock_probe;
+    if (!probe || threadIdx.x != 0) return;
+    const unsigned wg = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    if (wg >= (unsigned) CLOCK_PROBE_WORKGROUPS) return;
+    probe[4 * wg + 2 * at_end] = clock64();
+    probe[4 * wg + 2 * at_end + 1] = wall_clock64();
+}
+
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST>
+__device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
+{
+    // (a launch that its predicate skips leaves the cells to the launch that ran)
+    const bool probe = g.clock_probe && !(!CHK && g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0)));
+#ifdef MME_X_FROM
+    (void) probe;
+    gemm_fast_body_impl<ES, FMT, B_KC, AMODE, TM, RG, PERSIST, CHK, NST>(g);
+    PHASE(4);
+#else
+    if (probe) clock_probe_stamp(g, 0);
+    gemm_fast_body_impl<ES, FMT, B_KC, AMODE, TM, RG, PERSIST, CHK, NST>(g);
+    if (probe) clock_probe_stamp(g, 1);
+#endif
 }
 
 

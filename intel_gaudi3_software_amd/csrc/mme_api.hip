@@ -92,6 +92,9 @@ struct mme_hip_calc
     // device's static scratch array (noalloc_used: bytes handed out so far in this call)
     bool                  noalloc = false;
     size_t                noalloc_used = 0;
+    // diagnostics: per-workgroup clock stamps of the large-tile kernels (mme_hip_clock_probe), NULL while switched off
+    DeviceBuffer          clock_probe_buf;
+    uint64_t*             clock_probe = nullptr;
 };
 
 namespace
@@ -357,6 +360,7 @@ int plan_launch(mme_hip_handle h, GemmProblem& g)
     g.tile_m = gemm_fast_pick_tile_m(g, h->num_cus);
     g.split_k = gemm_pick_split_k(g, h->num_cus);
     g.workspace = nullptr;
+    g.clock_probe = h->clock_probe;
     if (g.split_k > 1)
     {
         void* ws = nullptr;
@@ -827,6 +831,84 @@ int mme_hip_set_wait_limit(mme_hip_handle h, unsigned polls)
 {
     if (!h) return MME_HIP_EINVAL;
     h->wait_limit = polls;
+    return MME_HIP_OK;
+}
+
+int mme_hip_clock_probe(mme_hip_handle h, int enable)
+{
+    if (!h) return MME_HIP_EINVAL;
+    h->clock_probe = nullptr;
+    if (!enable) return MME_HIP_OK;
+    const size_t bytes = (size_t) CLOCK_PROBE_WORKGROUPS * 4 * sizeof(uint64_t);
+    HIP_TRY(h, hipSetDevice(h->device));
+    HIP_TRY(h, h->clock_probe_buf.reserve(bytes));
+    HIP_TRY(h, launch_fill_u32((uint32_t*) h->clock_probe_buf.p, 0, bytes / 4, h->stream));
+    h->clock_probe = (uint64_t*) h->clock_probe_buf.p;
+    return MME_HIP_OK;
+}
+
+int mme_hip_clock_probe_read(mme_hip_handle h, double* shader_mhz, double* mean_us, double* max_us, int* workgroups)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (!h->clock_probe) return fail(h, MME_HIP_EINVAL, "mme_hip_clock_probe_read: the probe is switched off");
+    const size_t          cells = (size_t) CLOCK_PROBE_WORKGROUPS * 4;
+    std::vector<uint64_t> host(cells);
+    HIP_TRY(h, hipSetDevice(h->device));
+    HIP_TRY(h, hipMemcpyAsync(host.data(), h->clock_probe, cells * sizeof(uint64_t), hipMemcpyDeviceToHost, h->stream));
+    HIP_TRY(h, launch_fill_u32((uint32_t*) h->clock_probe, 0, cells * 2, h->stream));
+    HIP_TRY(h, hipStreamSynchronize(h->stream));
+    double clocks = 0, ticks = 0, worst = 0;
+    int    n = 0;
+    for (int wg = 0; wg < CLOCK_PROBE_WORKGROUPS; wg++)
+    {
+        const uint64_t* c = &host[4 * (size_t) wg];
+        if (!c[1] || c[3] <= c[1]) continue; // this workgroup did not run (or not to its end) since the last read
+        clocks += (double) (c[2] - c[0]);
+        ticks += (double) (c[3] - c[1]);
+        worst = std::max(worst, (double) (c[3] - c[1]));
+        n++;
+    }
+    if (workgroups) *workgroups = n;
+    if (shader_mhz) *shader_mhz = n ? clocks / ticks * 100.0 : 0.0;
+    if (mean_us) *mean_us = n ? ticks / n / 100.0 : 0.0;
+    if (max_us) *max_us = worst / 100.0;
+    return MME_HIP_OK;
+}
+
+int mme_hip_matrix_core_rate(mme_hip_handle h, int dtype, int random_operands, int iters, int launches, double* tflops, double* shader_mhz)
+{
+    if (!h || iters < 1 || launches < 1) return MME_HIP_EINVAL;
+    if (dtype != MME_HIP_FP8_143 && dtype != MME_HIP_BF16) return fail(h, MME_HIP_EUNSUPPORTED, "mme_hip_matrix_core_rate: fp8_143 or bf16");
+    const int kind = dtype == MME_HIP_FP8_143 ? 0 : 1;
+    HIP_TRY(h, hipSetDevice(h->device));
+    uint64_t* stamps = nullptr;
+    HIP_TRY(h, hipMalloc((void**) &stamps, 513 * sizeof(uint64_t)));
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t e = hipEventCreate(&e0);
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    for (int i = 0; i < 2 && e == hipSuccess; i++) e = launch_matrix_core_rate(kind, random_operands, iters, stamps, h->stream);
+    if (e == hipSuccess) e = hipEventRecord(e0, h->stream);
+    for (int i = 0; i < launches && e == hipSuccess; i++) e = launch_matrix_core_rate(kind, random_operands, iters, stamps, h->stream);
+    if (e == hipSuccess) e = hipEventRecord(e1, h->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(h->stream);
+    float                 ms = 0;
+    std::vector<uint64_t> host(512);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e == hipSuccess) e = hipMemcpy(host.data(), stamps, 512 * sizeof(uint64_t), hipMemcpyDeviceToHost);
+    if (e0) (void) hipEventDestroy(e0);
+    if (e1) (void) hipEventDestroy(e1);
+    (void) hipFree(stamps);
+    if (e != hipSuccess) return hip_fail(h, e, "mme_hip_matrix_core_rate");
+    double clocks = 0, ticks = 0;
+    for (int wg = 0; wg < 256; wg++)
+    {
+        clocks += (double) host[2 * wg];
+        ticks += (double) host[2 * wg + 1];
+    }
+    // 256 workgroups x 8 wavefronts x iters x 8 accumulators x one 32x32x64 step (fp8: one instruction, bf16: two of 32x32x16... x2)
+    const double flop_per_acc_step = kind == 0 ? 2.0 * 32 * 32 * 64 : 2.0 * 2.0 * 32 * 32 * 16;
+    if (tflops) *tflops = 256.0 * 8 * iters * 8 * flop_per_acc_step * launches / (ms * 1e-3) / 1e12;
+    if (shader_mhz) *shader_mhz = ticks > 0 ? clocks / ticks * 100.0 : 0.0;
     return MME_HIP_OK;
 }
 

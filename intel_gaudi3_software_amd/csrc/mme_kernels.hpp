@@ -138,7 +138,16 @@ struct GemmProblem
     // (mask 0: that operand needs no check).  The caller then enqueues the exact fall-back behind it, predicated on the flag.
     int             chk;
     uint32_t        chk_mask_a, chk_add_a, chk_mask_b, chk_add_b; // the byte constants replicated over a 32-bit word
+    // diagnostics (NULL: off): CLOCK_PROBE_WORKGROUPS x 4 cells in which the large-tile kernels note, per workgroup, the shader
+    // clock counter and the 100 MHz counter at its start and at its end
+    uint64_t*       clock_probe;
 };
+constexpr int CLOCK_PROBE_WORKGROUPS = 4096;
+
+// diagnostics: `iters` x 8 dependent-free 32x32 matrix instructions per wavefront on 256 workgroups of 8 wavefronts, operands in
+// registers (zero, or four sets of random codes used in turn); kind 0: fp8 (32x32x64), 1: bf16 (32x32x16).  stamps: 256 x 2
+// cells, shader clocks and 100 MHz ticks each workgroup's loop took.
+hipError_t launch_matrix_core_rate(int kind, int random_operands, int iters, uint64_t* stamps, hipStream_t s);
 
 size_t     gemm_workspace_bytes(const GemmProblem& p);
 int        gemm_pick_split_k(const GemmProblem& p, int num_cus);
