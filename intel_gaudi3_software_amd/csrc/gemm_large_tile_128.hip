@@ -11,22 +11,13 @@ namespace
 {
 // the fwd / dedx gather keeps six stages of 24 KiB in its ring (measured on the 3 x 3 dedx of 32 x 28 x 28 x 256: 3 % over four
 // stages; the plain GEMM and dedw, whose pipelines fill more slowly with a deeper ring, keep four)
-#ifndef MME_X_NSTC
-#define MME_X_NSTC 6
-#endif
-#ifndef MME_X_NSTG
-#define MME_X_NSTG 4
-#endif
-#ifndef MME_X_NSTW
-#define MME_X_NSTW 4
-#endif
-constexpr int NST128 = MME_X_NSTC, NSTG = MME_X_NSTG, NSTW = MME_X_NSTW;
+constexpr int NST128 = 6;
 
 template<int FMT, bool B_KC>
 __global__ __launch_bounds__(512) void gemm_2byte_fast128_kernel(GemmProblem g_by_value)
 {
     (void) g_by_value;
-    gemm_fast_body<2, FMT, B_KC, 0, 128, false, false, false, NSTG>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+    gemm_fast_body<2, FMT, B_KC, 0, 128>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
 }
 
 template<int FMT, bool B_KC>
@@ -40,7 +31,7 @@ template<int FMT>
 __global__ __launch_bounds__(512) void conv_dedw_2byte_fast128_kernel(GemmProblem g_by_value)
 {
     (void) g_by_value;
-    gemm_fast_body<2, FMT, false, 3, 128, false, false, false, NSTW>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+    gemm_fast_body<2, FMT, false, 3, 128>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
 }
 
 template<int FMT>
@@ -48,12 +39,12 @@ hipError_t launch_128(const GemmProblem& p, dim3 grid, hipStream_t s)
 {
     static bool attr_done[5] = {false, false, false, false, false};
     const bool  bkc = p.B.k_contig != 0;
-    if (p.A.kind == VIEW_CONV && !p.A.pix_is_f) return launch_fast(conv_dedw_2byte_fast128_kernel<FMT>, attr_done[4], p, grid, s, 128, NSTW);
+    if (p.A.kind == VIEW_CONV && !p.A.pix_is_f) return launch_fast(conv_dedw_2byte_fast128_kernel<FMT>, attr_done[4], p, grid, s, 128);
     if (p.A.kind == VIEW_CONV)
         return bkc ? launch_fast(conv_2byte_fast128_kernel<FMT, true>, attr_done[0], p, grid, s, 128, NST128)
                    : launch_fast(conv_2byte_fast128_kernel<FMT, false>, attr_done[1], p, grid, s, 128, NST128);
-    return bkc ? launch_fast(gemm_2byte_fast128_kernel<FMT, true>, attr_done[2], p, grid, s, 128, NSTG)
-               : launch_fast(gemm_2byte_fast128_kernel<FMT, false>, attr_done[3], p, grid, s, 128, NSTG);
+    return bkc ? launch_fast(gemm_2byte_fast128_kernel<FMT, true>, attr_done[2], p, grid, s, 128)
+               : launch_fast(gemm_2byte_fast128_kernel<FMT, false>, attr_done[3], p, grid, s, 128);
 }
 } // namespace
 

@@ -183,16 +183,9 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
 // NST: stages of the ring (default 4).  What a compute unit can draw from L2 / memory is the bytes it has in flight divided
 // by the latency, so a kernel whose stages are small (the 128-row tile: 24 KiB) keeps more of them in flight: six stages,
 // 144 KiB.  The reduction then has to be at least NST stages long.
-__device__ __forceinline__ void clock_probe_stamp(KARG GemmProblem& g, int at_end);
-#ifdef MME_X_FROM
-#define PHASE(k) do { if (g.clock_probe) { if (MME_X_FROM == (k)) clock_probe_stamp(g, 0); if (MME_X_TO == (k)) clock_probe_stamp(g, 1); } } while (0)
-#else
-#define PHASE(k) do { } while (0)
-#endif
 template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST>
 __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 {
-    PHASE(0);
     static_assert(NST >= 4 && NST <= 6 && (!PERSIST || NST == FNST), "ring depth");
     static_assert(!CHK || (ES == 1 && AMODE == 0 && TM == FBM && !RG), "operand checks: fp8, plain k-contiguous A, whole 256-row tiles");
     static_assert(!PERSIST || (AMODE == 0 && TM == FBM && !RG), "the persistent schedule: plain k-contiguous A, whole 256-row tiles");
@@ -529,7 +522,6 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             }
         }
     };
-    PHASE(1);
     issue_prologue();
     for (int walk_it = 0;;) // (one pass unless PERSIST)
     {
@@ -547,7 +539,6 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
                 for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
     }
     __syncthreads();
-    PHASE(2);
     auto read_a_any = [&](Frags & fr, int i, const char* st) __attribute__((always_inline))
     {
         if constexpr (A_KC) read_a(fr, i, st, wm * WR, lane);
@@ -556,22 +547,15 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         else
             read_a_tr16<TM>(fr, i, st, wm, lane);
     };
-    // The 128-row tile (two A fragments per wavefront) has registers to spare and only four matrix steps per stage to hide
-    // an LDS read behind: it keeps two fragment sets and fills the one for stage t+1 in one go at the start of step t, so no
-    // matrix instruction of a step waits for LDS.  The 256-row tile refills its single set register by register.
-#ifndef MME_X_DBUF
-#define MME_X_DBUF 1
-#endif
-    constexpr bool DBUF = NI == 2 && MME_X_DBUF;
-    Frags fr[DBUF ? 2 : 1];
+    Frags f;
 #pragma unroll
-    for (int i = 0; i < NI; i++) read_a_any(fr[0], i, lds);
+    for (int i = 0; i < NI; i++) read_a_any(f, i, lds);
 #pragma unroll
-    for (int j = 0; j < 2; j++) read_b(fr[0], j, lds);
+    for (int j = 0; j < 2; j++) read_b(f, j, lds);
 
     constexpr bool MSCALE = ES == 1 && AMODE == 0 && TM == FBM && !RG && !PERSIST && !CHK;
     const int      mfma_scale_a = 127 + (MSCALE ? g.epi.mfma_scale_exp : 0);
-    auto mma = [&](Frags & f, int i, int j) __attribute__((always_inline))
+    auto mma = [&](int i, int j) __attribute__((always_inline))
     {
         if constexpr (ES == 1)
         {
@@ -605,24 +589,15 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             }
         }
     };
-#ifndef MME_X_NOMMA
-#define MME_X_NOMMA 0
-#endif
-#ifndef MME_X_NOREAD
-#define MME_X_NOREAD 0
-#endif
-#ifndef MME_X_NODMA
-#define MME_X_NODMA 0
-#endif
-#define MMA(i, j) if (!MME_X_NOMMA) mma(fc, i, j)
+#define MMA(i, j) mma(i, j)
 #define RA(i) \
-    if (RN && !MME_X_NOREAD) read_a_any(fn, i, st);
+    if (RN) read_a_any(f, i, st);
 #define RB(j) \
-    if (RN && !MME_X_NOREAD) read_b(fn, j, st);
+    if (RN) read_b(f, j, st);
 #define LA(u) \
-    if (LOADS && !MME_X_NODMA) issue_a(u, t + NST, slot);
+    if (LOADS) issue_a(u, t + NST, slot);
 #define LB(u) \
-    if (LOADS && !MME_X_NODMA) issue_b(u, t + NST, slot);
+    if (LOADS) issue_b(u, t + NST, slot);
     // the look itself: this wavefront's eighth (2 KiB) of one operand's part of a stage, straight from LDS (the swizzled
     // placement does not matter, every byte of the part is an operand byte)
     auto chk_scan = [&](const char* part, uint32_t mask, uint32_t add) __attribute__((always_inline))
@@ -653,14 +628,11 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
     // other wavefront on the SIMD covers the tail of that latency); request stage t+4 into the slot of stage t, whose
     // fragments every wavefront read during the previous step (the barrier above orders those reads before this request).
-    auto step = [&](int t, auto waitc, auto loads, auto readnext, auto parity) __attribute__((always_inline))
+    auto step = [&](int t, auto waitc, auto loads, auto readnext) __attribute__((always_inline))
     {
         constexpr int  WAITC = decltype(waitc)::value;
         constexpr bool LOADS = decltype(loads)::value;
         constexpr bool RN = decltype(readnext)::value;
-        constexpr int  PAR = decltype(parity)::value; // t mod 2: which fragment set holds stage t (DBUF)
-        Frags&         fc = fr[DBUF ? PAR : 0];
-        Frags&         fn = fr[DBUF ? 1 - PAR : 0];
         const char*    st = lds + ((t + 1) % NST) * STAGE;
         const int      slot = t % NST;
         MMA(0, 0);
@@ -696,11 +668,10 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         }
         else
         {
-            // 128-row tile: four matrix steps per stage, three requests; all of stage t+1 goes to the other fragment set now
-            RA(0) RB(0) RA(1) RB(1) FENCE;
-            LA(0) LB(0) LB(1) FENCE;
-            MMA(1, 0); FENCE;
-            MMA(1, 1); FENCE;
+            // 128-row tile: four MFMAs per stage, three requests
+            RA(0) LA(0) MMA(1, 0); FENCE;
+            RB(0) LB(0) MMA(1, 1); FENCE;
+            RA(1) RB(1) LB(1) FENCE;
         }
     };
     // at the wait of step t the stages t+1 .. t+NST-1 have been requested; stage t+1 is needed, so the younger NST-2 stages of
@@ -708,34 +679,30 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     using WM = std::integral_constant<int, vm_wait((NST - 2) * NREQ)>;
     using T = std::true_type;
     using F = std::false_type;
-    using P0 = std::integral_constant<int, 0>;
-    using P1 = std::integral_constant<int, 1>;
     int t = 0;
     for (; t + NST + 1 < nk; t += 2) // steps 0 .. nk-NST-1 request stages NST .. nk-1
     {
-        step(t, WM {}, T {}, T {}, P0 {});
-        step(t + 1, WM {}, T {}, T {}, P1 {});
+        step(t, WM {}, T {}, T {});
+        step(t + 1, WM {}, T {}, T {});
     }
     if constexpr (NST % 2 != 0) // (the number of stages is even: an odd ring leaves one more step before the drain)
     {
-        step(t, WM {}, T {}, T {}, P0 {});
+        step(t, WM {}, T {}, T {});
         t++;
     }
-    constexpr int DP = NST % 2; // parity of the first step of the drain
     // t == nk - NST (nk >= NST): everything has been requested; step nk-NST+i needs stage nk-NST+i+1 with NST-2-i younger stages
     // behind it, the last step reads nothing
     auto drain = [&](auto ic) __attribute__((always_inline))
     {
         constexpr int I = decltype(ic)::value;
-        if constexpr (I < NST - 1)
-            step(t + I, std::integral_constant<int, vm_wait((NST - 2 - I) * NREQ)> {}, F {}, T {}, std::integral_constant<int, (DP + I) % 2> {});
+        if constexpr (I < NST - 1) step(t + I, std::integral_constant<int, vm_wait((NST - 2 - I) * NREQ)> {}, F {}, T {});
     };
     if constexpr (NST == 4)
     {
-        step(t, std::integral_constant<int, vm_wait(2 * NREQ)> {}, F {}, T {}, P0 {});
-        step(t + 1, std::integral_constant<int, vm_wait(NREQ)> {}, F {}, T {}, P1 {});
-        step(t + 2, std::integral_constant<int, vm_wait(0)> {}, F {}, T {}, P0 {});
-        step(t + 3, std::integral_constant<int, vm_wait(0)> {}, F {}, F {}, P1 {});
+        step(t, std::integral_constant<int, vm_wait(2 * NREQ)> {}, F {}, T {});
+        step(t + 1, std::integral_constant<int, vm_wait(NREQ)> {}, F {}, T {});
+        step(t + 2, std::integral_constant<int, vm_wait(0)> {}, F {}, T {});
+        step(t + 3, std::integral_constant<int, vm_wait(0)> {}, F {}, F {});
     }
     else
     {
@@ -744,9 +711,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         drain(std::integral_constant<int, 2> {});
         drain(std::integral_constant<int, 3> {});
         drain(std::integral_constant<int, 4> {});
-        step(t + NST - 1, std::integral_constant<int, vm_wait(0)> {}, F {}, F {}, std::integral_constant<int, (DP + NST - 1) % 2> {});
+        step(t + NST - 1, std::integral_constant<int, vm_wait(0)> {}, F {}, F {});
     }
-    PHASE(3);
 #undef MMA
 #undef RA
 #undef RB
@@ -1025,15 +991,9 @@ __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
     // (a launch that its predicate skips leaves the cells to the launch that ran)
     const bool probe = g.clock_probe && !(!CHK && g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0)));
-#ifdef MME_X_FROM
-    (void) probe;
-    gemm_fast_body_impl<ES, FMT, B_KC, AMODE, TM, RG, PERSIST, CHK, NST>(g);
-    PHASE(4);
-#else
     if (probe) clock_probe_stamp(g, 0);
     gemm_fast_body_impl<ES, FMT, B_KC, AMODE, TM, RG, PERSIST, CHK, NST>(g);
     if (probe) clock_probe_stamp(g, 1);
-#endif
 }
 
 
