@@ -16,7 +16,7 @@ void launch_gemm_fp8_11(const GemmProblem& p, dim3 grid, hipStream_t s);
 namespace
 {
 // sums the split-k partials in slice order (deterministic) and applies the epilogue.  Four consecutive columns per lane
-// (16-byte loads, one per slice, issued four slices at a time) when N is a multiple of 4; the sum of an element is formed
+// (16-byte loads, one per slice, up to sixteen slices in flight) when N is a multiple of 4; the sum of an element is formed
 // in the same order either way.
 __global__ __launch_bounds__(THREADS) void splitk_reduce_kernel(GemmProblem g_by_value)
 {
@@ -58,17 +58,17 @@ __global__ __launch_bounds__(THREADS) void splitk_reduce_kernel(GemmProblem g_by
             const r_v4f*    w = (const r_v4f*) (g.workspace + b * mn + r);
             const long long step = nb * mn / 4; // r_v4f elements between slices
             r_v4f           x = {0.0f, 0.0f, 0.0f, 0.0f};
-            int             z = 0;
-            for (; z + 4 <= S; z += 4)
+            // up to sixteen slices in flight per lane, added in slice order
+            for (int z0 = 0; z0 < S; z0 += 16)
             {
-                const r_v4f p0 = __builtin_nontemporal_load(w + (z + 0) * step), p1 = __builtin_nontemporal_load(w + (z + 1) * step),
-                            p2 = __builtin_nontemporal_load(w + (z + 2) * step), p3 = __builtin_nontemporal_load(w + (z + 3) * step);
-                x += p0;
-                x += p1;
-                x += p2;
-                x += p3;
+                r_v4f part[16];
+#pragma unroll
+                for (int j = 0; j < 16; j++)
+                    if (z0 + j < S) part[j] = __builtin_nontemporal_load(w + (z0 + j) * step);
+#pragma unroll
+                for (int j = 0; j < 16; j++)
+                    if (z0 + j < S) x += part[j];
             }
-            for (; z < S; z++) x += __builtin_nontemporal_load(w + z * step);
             const float xs[4] = {x.x, x.y, x.z, x.w};
             finish(b, r, 4, xs);
         }
@@ -228,7 +228,8 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s)
     if (p.split_k > 1)
     {
         const long long total = nb * p.M * (long long) p.N;
-        long long       blocks = (total + THREADS - 1) / THREADS;
+        const long long items = (p.N & 3) == 0 && ((uintptr_t) p.workspace & 15u) == 0 ? total >> 2 : total; // four columns per lane
+        long long       blocks = (items + THREADS - 1) / THREADS;
         if (blocks > 4096) blocks = 4096;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned) blocks), dim3(THREADS), 0, s, p);
         e = hipGetLastError();

@@ -246,7 +246,24 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     // workgroup ids are dealt round-robin to the 8 XCDs
     const int walk_first = PERSIST ? (int) ((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : 0;
     const int walk_total = PERSIST ? tiles_total * g.batch[0] * g.batch[1] * g.batch[2] : 0;
+    // split-k launches (grid = tiles x 1 x slices): the workgroups that land on one XCD (every eighth of the linear order) take
+    // consecutive (slice, tile) pairs, so the tiles of a k-slice, which all read the same slice of B and overlapping slices of
+    // A, find them in one L2 instead of fetching them into all eight
+    int kslice = 0, split_tile = (int) blockIdx.x;
+    if (!PERSIST && g.split_k > 1)
+    {
+        kslice = (int) blockIdx.z;
+        if (gridDim.y == 1)
+        {
+            const int total = (int) (gridDim.x * gridDim.z), lin = (int) (blockIdx.x + gridDim.x * blockIdx.z);
+            const int x = lin & 7, p = x * (total >> 3) + min(x, total & 7) + (lin >> 3); // a bijection of [0, total)
+            kslice = p / (int) gridDim.x;
+            split_tile = p - kslice * (int) gridDim.x;
+        }
+    }
     if constexpr (PERSIST) locate(walk_first % tiles_total, walk_first / tiles_total);
+    else if (g.split_k > 1)
+        locate(split_tile, blockIdx.y);
     else if ((tiles_m % 8 == 0) && (tiles_n % 4 == 0))
         locate((blockIdx.x & 7) * (tiles_total >> 3) + (blockIdx.x >> 3), blockIdx.y);
     else
@@ -261,8 +278,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    // split-k: blockIdx.z takes an equal slice of the stages and writes raw partial sums to the workspace
-    const int nk = g.K * ES / FBK / (g.split_k > 1 ? g.split_k : 1), kt_begin = (g.split_k > 1 ? (int) blockIdx.z : 0) * nk;
+    // split-k: slice `kslice` takes an equal share of the stages and writes raw partial sums to the workspace
+    const int nk = g.K * ES / FBK / (g.split_k > 1 ? g.split_k : 1), kt_begin = kslice * nk;
     // per-lane global pointers of this wavefront's 2 + 2 request slots (they advance by one stage per step)
     const uint8_t* ga[2];
     const uint8_t* gb[2];
@@ -852,7 +869,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     if (!PERSIST && g.split_k > 1)
     {
         // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
-        float* ws = g.workspace + ((long long) blockIdx.z * gridDim.y + blockIdx.y) * g.M * (long long) g.N + (long long) (em0 + ewm * WR) * g.N + en0 + ewn * 64;
+        float* ws = g.workspace + ((long long) kslice * gridDim.y + blockIdx.y) * g.M * (long long) g.N + (long long) (em0 + ewm * WR) * g.N + en0 + ewn * 64;
         walk_to(std::integral_constant<int, 4>(), std::true_type(), (uint8_t*) ws, (long long) g.N * 4, [&](const float (&val)[16], uint32_t (&pk)[16]) __attribute__((always_inline)) {
 #pragma unroll
             for (int c = 0; c < 16; c++) pk[c] = __float_as_uint(val[c]);
