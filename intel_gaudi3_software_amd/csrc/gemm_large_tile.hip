@@ -147,7 +147,7 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
         {
             // fwd / dedx: whole 64-byte stages inside one tap; the gather form of col2im only with unit strides; weights
             // plain or tapped (k-contiguous, same channel count)
-            if (p.A.nch % (FBK / es)) return false;
+            if (p.A.nch % (FBK / es) || p.A.nch * es > GF_ZERO_PAGE_BYTES) return false;
             for (int d = 0; d < 4; d++)
                 if (p.A.gather_y && p.A.cstride[d] != 1) return false;
             if (p.B.kind == VIEW_TAPPED && (!p.B.k_contig || p.B.nch != p.A.nch || p.B.stride_k != 1)) return false;

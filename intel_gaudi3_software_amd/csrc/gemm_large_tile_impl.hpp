@@ -157,7 +157,7 @@ __device__ __forceinline__ void warm_kernargs(KARG GemmProblem& g)
 // forward pass, its gather-form inverse for dedx): row r of the tile is a pixel, a 64-byte stage is a run of channels
 // of one filter tap, so a request's address is (pixel's offset for tap 0) + (the tap's uniform offset) + channel, or a
 // page of zeros where the tap falls outside the source tensor.  B may then be a tapped weight view (dedx).
-__device__ __attribute__((aligned(16))) uint32_t gf_zero_page[4];
+__device__ __attribute__((aligned(16))) uint32_t gf_zero_page[GF_ZERO_PAGE_BYTES / 4];
 
 //
 // AMODE says how operand A is addressed: 0 plain, k contiguous; 1 convolution view with pixels along f (GATHER above);
@@ -332,15 +332,36 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     uint32_t  tap_ok[2] = {0, 0};      // bit t: tap t of this lane's row (request slot u) reads inside the source tensor
     int       g_tap = 0, g_ch = 0;     // uniform: tap and first channel of the next stage to request
     int       g_t[3] = {0, 0, 0};      // g_tap as (s, r, q)
-    long long g_delta_a = 0, g_delta_b = 0; // uniform byte offsets of that stage: tap offset + channel
+    int       g_chb = 0;               // uniform: g_ch in bytes
+    long long g_delta_b = 0;           // uniform byte offset of that stage in the weights (tapped: tap + channel; plain: stage)
+    long long g_step_b = 0;            // plain weights: bytes from one stage to the next
+    // per lane and request slot: where the current tap's channels of this lane's row start, or the zero page when the tap
+    // falls into the padding (the zero page is as long as a row's channels, so every lane adds the same channel offset)
+    const uint8_t* a_tap[2] = {nullptr, nullptr};
     const int stage_ch = FBK / ES;     // channels per stage
-    auto      gather_offsets = [&]() __attribute__((always_inline))
+    // (values that are the same in every lane are handed back to scalar registers after the vector arithmetic of a tap change)
+    auto uniform32 = [](int x) __attribute__((always_inline)) { return __builtin_amdgcn_readfirstlane(x); };
+    auto uniform64 = [](long long x) __attribute__((always_inline))
+    {
+        const uint32_t lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) x), hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) ((unsigned long long) x >> 32));
+        return (long long) (((unsigned long long) hi << 32) | lo);
+    };
+    // a new tap (once per nch / stage_ch stages): its offset in the gathered tensor and in the tapped weights, and every
+    // lane's base address for it
+    auto gather_offsets = [&]() __attribute__((always_inline))
     {
         long long d = 0;
 #pragma unroll
         for (int q = 0; q < 3; q++) d += (long long) g_t[q] * g.A.dil[q] * g.A.src_stride[q];
-        g_delta_a = ((g.A.gather_y ? -d : d) + g_ch) * ES;
-        g_delta_b = ((long long) g_tap * g.B.tap_stride + g_ch) * ES;
+        const long long tap_a = uniform64((g.A.gather_y ? -d : d) * ES);
+        if (g.B.kind == VIEW_TAPPED) g_delta_b = uniform64(((long long) g_tap * g.B.tap_stride + g_ch) * ES);
+        g_chb = uniform32(g_ch * ES);
+#pragma unroll
+        for (int u = 0; u < NUA; u++)
+        {
+            const bool ok = (tap_ok[u] >> g_tap) & 1u;
+            a_tap[u] = ok ? ga[u] + tap_a : (const uint8_t*) gf_zero_page;
+        }
     };
     auto gather_advance = [&]() __attribute__((always_inline))
     {
@@ -348,7 +369,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         if (g_ch >= g.A.nch)
         {
             g_ch = 0;
-            g_tap++;
+            g_tap = uniform32(g_tap + 1);
             if (++g_t[0] == g.A.ktap[0])
             {
                 g_t[0] = 0;
@@ -358,14 +379,18 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
                     g_t[2]++;
                 }
             }
+#pragma unroll
+            for (int q = 0; q < 3; q++) g_t[q] = uniform32(g_t[q]);
             gather_offsets();
         }
         else
         {
             // same tap, next channels: the common case costs two scalar additions
-            g_delta_a += FBK;
-            g_delta_b += FBK;
+            g_chb += FBK;
+            if (g.B.kind == VIEW_TAPPED) g_delta_b += FBK;
         }
+        // (plain weights: the stage's offset does not depend on the tap)
+        if (g.B.kind != VIEW_TAPPED) g_delta_b += g_step_b;
     };
     if constexpr (GATHER)
     {
@@ -420,6 +445,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         const int k0 = kt_begin * stage_ch;
         g_tap = k0 / g.A.nch;
         g_ch = k0 - g_tap * g.A.nch;
+        g_step_b = uniform64(B_KC ? (long long) FBK : (long long) (FBK / ES) * ldb);
+        g_delta_b = 0; // (plain weights: gb[u] points at this workgroup's first stage)
         g_t[0] = g_tap % g.A.ktap[0];
         g_t[1] = (g_tap / g.A.ktap[0]) % g.A.ktap[1];
         g_t[2] = g_tap / (g.A.ktap[0] * g.A.ktap[1]);
@@ -498,23 +525,21 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             dma16(ga[u] + (size_t) stage * (FBK / ES) * lda, lds_base + slot * STAGE + (wave * 2 + u) * 1024);
         else if constexpr (GATHER)
         {
-            const bool     ok = (tap_ok[u] >> g_tap) & 1u;
-            const uint8_t* src = ok ? ga[u] + g_delta_a : zero_page();
-            dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
+            dma16(a_tap[u] + g_chb, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
         }
         else
             dma16(ga[u] + (size_t) stage * FBK, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
     };
     auto issue_b = [&](int u, int stage, int slot) __attribute__((always_inline))
     {
-        if (GATHER && g.B.kind == VIEW_TAPPED)
+        if constexpr (GATHER)
         {
+            // one running offset for both kinds of weights, so the step has no branch on the kind
             dma16(gb[u] + g_delta_b, lds_base + slot * STAGE + A_BYTES + (wave * 2 + u) * 1024);
             if (u == 1) gather_advance(); // the stage's last request
             return;
         }
         dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * STAGE + A_BYTES + (wave * 2 + u) * 1024);
-        if (GATHER && u == 1) gather_advance();
     };
     auto read_b = [&](Frags & f, int j, const char* st) __attribute__((always_inline))
     {
@@ -645,13 +670,27 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
     // other wavefront on the SIMD covers the tail of that latency); request stage t+4 into the slot of stage t, whose
     // fragments every wavefront read during the previous step (the barrier above orders those reads before this request).
+    int  slot_of_step = 0; // t mod NST of the next step
     auto step = [&](int t, auto waitc, auto loads, auto readnext) __attribute__((always_inline))
     {
         constexpr int  WAITC = decltype(waitc)::value;
         constexpr bool LOADS = decltype(loads)::value;
         constexpr bool RN = decltype(readnext)::value;
-        const char*    st = lds + ((t + 1) % NST) * STAGE;
-        const int      slot = t % NST;
+        // slots of stage t (to be refilled) and of stage t+1 (to be read): the steps run in order from t = 0, so a ring whose
+        // depth is not a power of two counts its slots up instead of dividing
+        int slot, next_slot;
+        if constexpr ((NST & (NST - 1)) == 0)
+        {
+            slot = t % NST;
+            next_slot = (t + 1) % NST;
+        }
+        else
+        {
+            slot = slot_of_step;
+            next_slot = slot_of_step + 1 == NST ? 0 : slot_of_step + 1;
+            slot_of_step = next_slot;
+        }
+        const char* st = lds + next_slot * STAGE;
         MMA(0, 0);
         FENCE;
         if (RN)

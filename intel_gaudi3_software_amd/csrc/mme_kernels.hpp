@@ -143,6 +143,9 @@ struct GemmProblem
     uint64_t*       clock_probe;
 };
 constexpr int CLOCK_PROBE_WORKGROUPS = 4096;
+// the page of zeros that the convolution gathers of the large-tile kernels read where a filter tap falls into the padding: as long
+// as the channels of one tap may be (a padding lane adds the stage's channel offset like every other lane)
+constexpr int GF_ZERO_PAGE_BYTES = 4096;
 
 // diagnostics: `iters` x 8 dependent-free 32x32 matrix instructions per wavefront on 256 workgroups of 8 wavefronts, operands in
 // registers (zero, or four sets of random codes used in turn); kind 0: fp8 (32x32x64), 1: bf16 (32x32x16).  stamps: 256 x 2
