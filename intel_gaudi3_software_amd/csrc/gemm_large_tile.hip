@@ -157,6 +157,9 @@ bool gemm_large_tile_applicable(const GemmProblem& p)
         {
             // dedw: 16-byte chunks of channels inside one tap, dY plain with its channels contiguous
             if (p.A.gather_y || p.A.nch % (16 / es) || p.B.kind != VIEW_PLAIN || p.B.k_contig) return false;
+            // (the kernel keeps the source tensor's strides in bytes in 32-bit registers)
+            for (int d = 0; d < 4; d++)
+                if (p.A.src_stride[d] < 0 || p.A.src_stride[d] * es >= (1ll << 32)) return false;
         }
     }
     else if (p.A.kind != VIEW_PLAIN || p.B.kind != VIEW_PLAIN)

@@ -454,13 +454,31 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     }
     // ---- AMODE 3: this lane's (tap, channel) per request slot and the pixel of the next stage to request -----------------
     int       w_pc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}}; // pixel coordinates (dims 1..4 of the tensor that enumerates pixels)
-    int       w_t[2][3] = {{0, 0, 0}, {0, 0, 0}};        // tap as (s, r, q)
-    long long w_ch[2] = {0, 0};                          // channel byte offset, < 0: f beyond M
+    int       w_tc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}}; // this lane's tap in the source tensor's coordinates: tap * dilation - padding
+    int       w_chb[2] = {0, 0};                         // channel byte offset, < 0: f beyond M
     float     w_rcp[3] = {0.0f, 0.0f, 0.0f};             // 1 / grid[d]
+    // what every request of the loop needs of the problem description, read once and pinned in scalar registers (a read
+    // inside a step would wait on the counter that the step's LDS reads share): the convolution strides, the source
+    // tensor's extents and its strides in bytes (below 2^32, the host sees to that) and the extents of the pixel grid
+    int      w_cs[4] = {0, 0, 0, 0}, w_src[4] = {0, 0, 0, 0}, w_grid[3] = {0, 0, 0};
+    uint32_t w_sb[4] = {0, 0, 0, 0};
     if constexpr (AMODE == 3)
     {
 #pragma unroll
-        for (int d = 0; d < 3; d++) w_rcp[d] = __builtin_amdgcn_rcpf((float) g.A.grid[d]);
+        for (int d = 0; d < 4; d++)
+        {
+            w_cs[d] = g.A.cstride[d];
+            w_src[d] = g.A.src[d];
+            w_sb[d] = (uint32_t) (g.A.src_stride[d] * ES);
+            asm volatile("" : "+s"(w_cs[d]), "+s"(w_src[d]), "+s"(w_sb[d]));
+        }
+#pragma unroll
+        for (int d = 0; d < 3; d++)
+        {
+            w_grid[d] = g.A.grid[d];
+            asm volatile("" : "+s"(w_grid[d]));
+            w_rcp[d] = __builtin_amdgcn_rcpf((float) w_grid[d]);
+        }
 #pragma unroll
         for (int u = 0; u < 2; u++)
         {
@@ -470,10 +488,11 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             // 16-byte chunk of the row that this lane fetches (the swizzles of the two stage layouts)
             const int chunk = ES == 1 ? ((lane & 15) - 2 * (kr & 7)) & 15 : (lane & (64 / RPQ - 1)) ^ ((kr & 3) << 1);
             const int f = m0 + chunk * (16 / ES), tap = f / g.A.nch;
-            w_ch[u] = f < g.M ? (long long) (f - tap * g.A.nch) * ES : -1;
-            w_t[u][0] = tap % g.A.ktap[0];
-            w_t[u][1] = (tap / g.A.ktap[0]) % g.A.ktap[1];
-            w_t[u][2] = tap / (g.A.ktap[0] * g.A.ktap[1]);
+            w_chb[u] = f < g.M ? (f - tap * g.A.nch) * ES : -1;
+            w_tc[u][0] = (tap % g.A.ktap[0]) * g.A.dil[0] - g.A.pad[0];
+            w_tc[u][1] = ((tap / g.A.ktap[0]) % g.A.ktap[1]) * g.A.dil[1] - g.A.pad[1];
+            w_tc[u][2] = (tap / (g.A.ktap[0] * g.A.ktap[1])) * g.A.dil[2] - g.A.pad[2];
+            w_tc[u][3] = -g.A.pad[3];
             const PixelPos pp = decode_pixel(g.A, kt_begin * (FBK / ES) + kr);
 #pragma unroll
             for (int d = 0; d < 4; d++) w_pc[u][d] = pp.c[d];
@@ -495,14 +514,16 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         if constexpr (AMODE == 3)
         {
             // x[pos(pixel, tap)][channel .. + 7], or zeros where the tap falls into the padding
-            long long off = w_ch[u];
-            bool      ok = off >= 0;
+            // (a position outside the tensor fails the unsigned comparison whether it is negative or too large; its offset is
+            // then not used)
+            uint64_t off = (uint64_t) (uint32_t) w_chb[u];
+            bool     ok = w_chb[u] >= 0;
 #pragma unroll
             for (int d = 0; d < 4; d++)
             {
-                const int pos = w_pc[u][d] * g.A.cstride[d] + (d < 3 ? w_t[u][d] * g.A.dil[d] : 0) - g.A.pad[d];
-                ok = ok && pos >= 0 && pos < g.A.src[d];
-                off += (long long) pos * g.A.src_stride[d] * ES;
+                const int pos = w_pc[u][d] * w_cs[d] + w_tc[u][d];
+                ok = ok && (uint32_t) pos < (uint32_t) w_src[d];
+                off += (uint64_t) (uint32_t) pos * w_sb[d];
             }
             const uint8_t* src = ok ? A + off : zero_page();
             dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
@@ -512,7 +533,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             for (int d = 0; d < 3; d++)
             {
                 // v / grid[d] for small non-negative v: float estimate, corrected by one
-                const int v = w_pc[u][d] + carry, gd = g.A.grid[d];
+                const int v = w_pc[u][d] + carry, gd = w_grid[d];
                 int       q = (int) ((float) v * w_rcp[d]);
                 const int r = v - q * gd;
                 q += (r >= gd) - (r < 0);
