@@ -456,7 +456,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     int       w_pc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}}; // pixel coordinates (dims 1..4 of the tensor that enumerates pixels)
     int       w_tc[2][4] = {{0, 0, 0, 0}, {0, 0, 0, 0}}; // this lane's tap in the source tensor's coordinates: tap * dilation - padding
     int       w_chb[2] = {0, 0};                         // channel byte offset, < 0: f beyond M
-    float     w_rcp[3] = {0.0f, 0.0f, 0.0f};             // 1 / grid[d]
+    int       w_step[4] = {0, 0, 0, 0};                  // the pixels of one stage as digits in the radix of the pixel grid
     // what every request of the loop needs of the problem description, read once and pinned in scalar registers (a read
     // inside a step would wait on the counter that the step's LDS reads share): the convolution strides, the source
     // tensor's extents and its strides in bytes (below 2^32, the host sees to that) and the extents of the pixel grid
@@ -477,7 +477,18 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         {
             w_grid[d] = g.A.grid[d];
             asm volatile("" : "+s"(w_grid[d]));
-            w_rcp[d] = __builtin_amdgcn_rcpf((float) w_grid[d]);
+        }
+        {
+            int rest = FBK / ES;
+#pragma unroll
+            for (int d = 0; d < 3; d++)
+            {
+                w_step[d] = __builtin_amdgcn_readfirstlane(rest % w_grid[d]);
+                rest = __builtin_amdgcn_readfirstlane(rest / w_grid[d]);
+            }
+            w_step[3] = rest;
+#pragma unroll
+            for (int d = 0; d < 4; d++) asm volatile("" : "+s"(w_step[d]));
         }
 #pragma unroll
         for (int u = 0; u < 2; u++)
@@ -527,20 +538,17 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             }
             const uint8_t* src = ok ? A + off : zero_page();
             dma16(src, lds_base + slot * STAGE + (wave * NUA + u) * 1024);
-            // next stage: 32 (2-byte elements) or 64 (fp8) pixels further
-            int carry = FBK / ES;
+            // next stage: 32 (2-byte elements) or 64 (fp8) pixels further, added digit by digit in the mixed radix of the pixel
+            // grid (a digit of the step is smaller than its radix, so one conditional subtraction per digit is enough)
+            int carry = 0;
 #pragma unroll
             for (int d = 0; d < 3; d++)
             {
-                // v / grid[d] for small non-negative v: float estimate, corrected by one
-                const int v = w_pc[u][d] + carry, gd = w_grid[d];
-                int       q = (int) ((float) v * w_rcp[d]);
-                const int r = v - q * gd;
-                q += (r >= gd) - (r < 0);
-                carry = q;
-                w_pc[u][d] = v - q * gd;
+                const int v = w_pc[u][d] + w_step[d] + carry;
+                carry = v >= w_grid[d] ? 1 : 0;
+                w_pc[u][d] = v - (carry ? w_grid[d] : 0);
             }
-            w_pc[u][3] += carry;
+            w_pc[u][3] += w_step[3] + carry;
         }
         else if constexpr (AMODE == 2)
             dma16(ga[u] + (size_t) stage * (FBK / ES) * lda, lds_base + slot * STAGE + (wave * 2 + u) * 1024);
