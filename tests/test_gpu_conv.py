@@ -279,6 +279,16 @@ GATHER_CASES = [
 ]
 
 
+# the gather's padding lanes read a page of zeros as long as a tap's channels may be (4096 bytes): 2048 bf16 channels still
+# take the large-tile kernel (every lane of a padded tap walks to the page's last 64 bytes), 2112 are routed to the general
+# kernel; the gathered tensor is x for fwd (C channels) and dy for dedx (K channels)
+@pytest.mark.parametrize("op,C,K", [(abi.OP_FWD, 2048, 128), (abi.OP_FWD, 2112, 128), (abi.OP_DEDX, 128, 2048), (abi.OP_DEDX, 128, 2112)])
+def test_conv_gather_with_as_many_channels_as_the_zero_page_holds(calc, orc, op, C, K):
+    case = (C, K, 6, 5, 1, 1, 3, 3, 1, (1, 1, 0), (1, 1, 1), (1, 1, 1), 2)
+    got, want = _run(calc, orc, case, abi.BF16, 0, op, device=True)
+    assert rel_frobenius(got, want) <= 1e-4
+
+
 @pytest.mark.parametrize("case", GATHER_CASES)
 @pytest.mark.parametrize("op", [abi.OP_FWD, abi.OP_DEDX])
 @pytest.mark.parametrize("dt,bias", [(abi.BF16, 0), (abi.FP16, 15), (abi.FP16, 11), (abi.FP8_143, 7), (abi.FP8_143, 11), (abi.FP8_152, 15)])
