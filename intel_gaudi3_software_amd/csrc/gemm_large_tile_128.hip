@@ -9,10 +9,6 @@ namespace mme
 {
 namespace
 {
-// the fwd / dedx gather keeps six stages of 24 KiB in its ring (measured on the 3 x 3 dedx of 32 x 28 x 28 x 256: 3 % over four
-// stages; the plain GEMM and dedw, whose pipelines fill more slowly with a deeper ring, keep four)
-constexpr int NST128 = 6;
-
 template<int FMT, bool B_KC>
 __global__ __launch_bounds__(512) void gemm_2byte_fast128_kernel(GemmProblem g_by_value)
 {
@@ -24,7 +20,7 @@ template<int FMT, bool B_KC>
 __global__ __launch_bounds__(512) void conv_2byte_fast128_kernel(GemmProblem g_by_value)
 {
     (void) g_by_value;
-    gemm_fast_body<2, FMT, B_KC, 1, 128, false, false, false, NST128>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
+    gemm_fast_body<2, FMT, B_KC, 1, 128>(*(KARG GemmProblem*) __builtin_amdgcn_kernarg_segment_ptr());
 }
 
 template<int FMT>
@@ -41,8 +37,8 @@ hipError_t launch_128(const GemmProblem& p, dim3 grid, hipStream_t s)
     const bool  bkc = p.B.k_contig != 0;
     if (p.A.kind == VIEW_CONV && !p.A.pix_is_f) return launch_fast(conv_dedw_2byte_fast128_kernel<FMT>, attr_done[4], p, grid, s, 128);
     if (p.A.kind == VIEW_CONV)
-        return bkc ? launch_fast(conv_2byte_fast128_kernel<FMT, true>, attr_done[0], p, grid, s, 128, NST128)
-                   : launch_fast(conv_2byte_fast128_kernel<FMT, false>, attr_done[1], p, grid, s, 128, NST128);
+        return bkc ? launch_fast(conv_2byte_fast128_kernel<FMT, true>, attr_done[0], p, grid, s, 128)
+                   : launch_fast(conv_2byte_fast128_kernel<FMT, false>, attr_done[1], p, grid, s, 128);
     return bkc ? launch_fast(gemm_2byte_fast128_kernel<FMT, true>, attr_done[2], p, grid, s, 128)
                : launch_fast(gemm_2byte_fast128_kernel<FMT, false>, attr_done[3], p, grid, s, 128);
 }

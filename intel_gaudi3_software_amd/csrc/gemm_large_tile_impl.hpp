@@ -180,9 +180,9 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[GF_ZERO_PAGE_BYTES
 // the A rows by the tile column t mod tiles_n, of the B columns by the tile row t mod tiles_m): when its turn comes, each
 // wavefront reads an eighth of that part of the stage once more from LDS and tests the bytes, a few vector instructions in
 // the shadow of the matrix instructions, so a clean operand costs no extra pass over memory and no extra launch.
-// NST: stages of the ring (default 4).  What a compute unit can draw from L2 / memory is the bytes it has in flight divided
-// by the latency, so a kernel whose stages are small (the 128-row tile: 24 KiB) keeps more of them in flight: six stages,
-// 144 KiB.  The reduction then has to be at least NST stages long.
+// NST: stages of the ring (4 to 6, default 4; every instantiation uses the default: six stages of the 128-row tile's 24 KiB
+// measured 2-3 % slower than four on the 3 x 3 convolutions of 32 x 28 x 28 x 256, whose steps then divide by six to find a slot).
+// The reduction has to be at least NST stages long.
 template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST>
 __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 {
