@@ -765,7 +765,18 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     using T = std::true_type;
     using F = std::false_type;
     int t = 0;
-    for (; t + NST + 1 < nk; t += 2) // steps 0 .. nk-NST-1 request stages NST .. nk-1
+    // steps 0 .. nk-NST-1 request stages NST .. nk-1.  The 128-row tile walks the four-stage ring four steps at a time: t is
+    // then a multiple of four, the slots of a step are compile-time constants and the LDS addresses of its reads and
+    // requests need no arithmetic; what is left of the steps (a pair, the count is even) follows.
+    if constexpr (TM == 128 && NST == 4 && !PERSIST)
+        for (; t + NST + 3 < nk; t += 4)
+        {
+            step(t, WM {}, T {}, T {});
+            step(t + 1, WM {}, T {}, T {});
+            step(t + 2, WM {}, T {}, T {});
+            step(t + 3, WM {}, T {}, T {});
+        }
+    for (; t + NST + 1 < nk; t += 2)
     {
         step(t, WM {}, T {}, T {});
         step(t + 1, WM {}, T {}, T {});
