@@ -28,6 +28,10 @@ def build(with_ref=True):
     if with_ref and os.path.isdir(os.environ.get("MME_REFERENCE_ROOT", "/root/reference")):
         subprocess.check_call(["make", "-s", "-j8", "-C", _HERE, "ref",
                                "REF=" + os.environ.get("MME_REFERENCE_ROOT", "/root/reference")])
+        # the drop-in demonstration links the MI355X library: built only where that has been built
+        if os.path.exists(os.path.join(_HERE, "..", "intel_gaudi3_software_amd", "csrc", "libmme_hip.so")):
+            subprocess.check_call(["make", "-s", "-j8", "-C", _HERE, "ref_dropin",
+                                   "REF=" + os.environ.get("MME_REFERENCE_ROOT", "/root/reference")])
 
 
 def oracle():
