@@ -31,9 +31,11 @@ PEAK_TFLOPS = {"fp8": 5000.0, "bf16": 2500.0, "fp32": 157.3}  # dense MFMA peaks
 PEAK_HBM_GBS = 8000.0
 METRIC = "TFLOP/s & % fp8/bf16 MFMA peak (GEMM, conv); cast GB/s vs HBM peak; 1 GPU"
 
-# HBM bytes per launch of the fp8 GEMM kernel on this workload, from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-# profiles/gemm_fp8_fast_kernel_4096x4096x4096_hbm_traffic.txt (96.3 MiB fetched + 32.1 MiB written; 64 MiB algorithmic)
+# HBM bytes per launch of each workload's kernels (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter runs
+# summarised per workload under profiles/ (the headline GEMM: 101.0 MB fetched + 33.6 MB written for 67.1 MB algorithmic)
 GEMM_TRAFFIC_BYTES = 134.6e6
+TRAFFIC_BYTES = {"c1": 4.4e6, "c3": 54.9e6, "c4_dedx": 54.0e6, "c4_dedw": 71.9e6 + 35.5e6, "c5": 844.3e6, "cast_fp8_143": 1342.1e6,
+                 "cast_bf16": 1610.6e6, "dequant_fp8_143": 1342.4e6}
 
 SECONDARY = ("c1", "c3", "c4_dedx", "c4_dedw", "c5", "cast_fp8_143", "cast_bf16", "dequant_fp8_143")
 
@@ -575,7 +577,9 @@ def main():
         if args.only not in WORKLOADS:
             print("unknown workload %r" % args.only, file=sys.stderr)
             sys.exit(2)
-        print(json.dumps({args.only: WORKLOADS[args.only](b)}))
+        res = WORKLOADS[args.only](b)
+        res["roofline"]["traffic"] = TRAFFIC_BYTES.get(args.only)
+        print(json.dumps({args.only: res}))
         b.calc.close()
         return
     result = run_c2(b)
@@ -583,6 +587,7 @@ def main():
         result["secondary"] = {}
         for name in SECONDARY:
             result["secondary"][name] = WORKLOADS[name](b)
+            result["secondary"][name]["roofline"]["traffic"] = TRAFFIC_BYTES.get(name)
             b.torch.cuda.empty_cache()
     if args.extra:
         result["extra"] = extra_measurements(b.calc, b.stream)
