@@ -239,8 +239,14 @@ int mme_hip_set_wait_limit(mme_hip_handle h, unsigned polls);
  * for MME_HIP_FP8_143, 32x32x16 for MME_HIP_BF16) on every compute unit, operands in registers, all zero or
  * (random_operands != 0) random and changing from instruction to instruction: the rate the matrix cores sustain on this
  * device with nothing else to do, and the clock they held.
+ *
+ * mme_hip_last_contraction_form: which form of the contraction kernels the latest doBatchGemm / doConvolution call of this
+ * handle launched: large_tile 1 when a large-tile kernel took it (0: the general kernel), the rows of its output tile (256 or
+ * 128), the slices of the reduction (1: no split-k) and the wavefronts per workgroup (8, or 4 for the fp8 GEMM form with
+ * 128 x 128 outputs per wavefront).  Lets a test state which kernel it is about.
  */
 int mme_hip_clock_probe(mme_hip_handle h, int enable);
+int mme_hip_last_contraction_form(mme_hip_handle h, int* large_tile, int* tile_rows, int* split_k, int* wavefronts);
 int mme_hip_clock_probe_read(mme_hip_handle h, double* shader_mhz, double* mean_us, double* max_us, int* workgroups);
 int mme_hip_matrix_core_rate(mme_hip_handle h, int dtype, int random_operands, int iters, int launches, double* tflops, double* shader_mhz);
 

@@ -139,6 +139,7 @@ def load_library():
     L.mme_hip_set_wait_limit.argtypes = [vp, C.c_uint]
     L.mme_hip_clock_probe.argtypes = [vp, C.c_int]
     L.mme_hip_clock_probe_read.argtypes = [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int)]
+    L.mme_hip_last_contraction_form.argtypes = [vp] + [C.POINTER(C.c_int)] * 4
     L.mme_hip_matrix_core_rate.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.mme_hip_set_fp8_specials_policy.argtypes = [vp, C.c_int]
     L.mme_hip_set_operand_clip.argtypes = [vp, C.c_int, C.c_int]

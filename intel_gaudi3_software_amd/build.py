@@ -5,7 +5,7 @@ import sys
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
-SOURCES = ["cast_kernels.hip", "gemm_kernels.hip", "gemm_inst_bf16.hip", "gemm_inst_fp16.hip", "gemm_inst_fp32.hip", "gemm_inst_fp8_00.hip", "gemm_inst_fp8_10.hip", "gemm_inst_fp8_01.hip", "gemm_inst_fp8_11.hip", "gemm_large_tile.hip", "gemm_large_tile_f16.hip", "gemm_large_tile_128.hip", "gemm_large_tile_ragged.hip", "gemm_large_tile_conv_fp8.hip", "gemm_large_tile_fp8_at.hip", "gemm_large_tile_ragged_conv.hip", "gemm_large_tile_persistent.hip", "gemm_large_tile_chk.hip", "gemm_large_tile_persistent_chk.hip", "conv_fwd_fast.hip", "diagnostics.hip", "mme_api.hip"]
+SOURCES = ["cast_kernels.hip", "gemm_kernels.hip", "gemm_inst_bf16.hip", "gemm_inst_fp16.hip", "gemm_inst_fp32.hip", "gemm_inst_fp8_00.hip", "gemm_inst_fp8_10.hip", "gemm_inst_fp8_01.hip", "gemm_inst_fp8_11.hip", "gemm_large_tile.hip", "gemm_large_tile_f16.hip", "gemm_large_tile_128.hip", "gemm_large_tile_ragged.hip", "gemm_large_tile_conv_fp8.hip", "gemm_large_tile_fp8_at.hip", "gemm_large_tile_ragged_conv.hip", "gemm_large_tile_persistent.hip", "gemm_large_tile_chk.hip", "gemm_large_tile_persistent_chk.hip", "gemm_large_tile_w4.hip", "conv_fwd_fast.hip", "diagnostics.hip", "mme_api.hip"]
 LIB = os.path.join(CSRC, "libmme_hip.so")
 
 # -packed-fp32-ops is switched off: some packed fp32 forms have produced wrong results on this hardware pool

@@ -261,6 +261,14 @@ class HipCalculator:
         self._in_flight.clear()
         return {"shader_mhz": mhz.value, "workgroup_us_mean": mean.value, "workgroup_us_max": worst.value, "workgroups": n.value}
 
+    def lastContractionForm(self):
+        """Which kernel form the latest doBatchGemm / doConvolution launched (mme_hip_last_contraction_form):
+        {large_tile, tile_rows, split_k, wavefronts}."""
+        import ctypes as C
+        v = [C.c_int() for _ in range(4)]
+        self._check(self._lib.mme_hip_last_contraction_form(self._h, *[C.byref(x) for x in v]))
+        return {"large_tile": bool(v[0].value), "tile_rows": v[1].value, "split_k": v[2].value, "wavefronts": v[3].value}
+
     def matrixCoreRate(self, dtype, random_operands, iters=4096, launches=10):
         """(TFLOP/s, shader clock in MHz) of back-to-back matrix instructions with operands in registers
         (mme_hip_matrix_core_rate): what the matrix cores sustain on this device and this kind of data."""

@@ -27,23 +27,27 @@ __device__ __forceinline__ void dma16(const void* g, uint32_t lds_off)
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_off) : "memory");
 }
 
-struct Frags
+// operand fragments of one stage: four 32-row blocks of A, NJ 32-column blocks of B
+template<int NJ>
+struct FragsT
 {
-    v8i a[4], b[2];
+    v8i a[4], b[NJ];
 };
 
 // (row0: first row of this wavefront's block of the staged A tile; the B readers take the address of the stage's B part)
-__device__ __forceinline__ void read_a(Frags& f, int i, const char* st, int row0, int lane)
+template<class FR>
+__device__ __forceinline__ void read_a(FR& f, int i, const char* st, int row0, int lane)
 {
     const int r = row0 + i * 32 + (lane & 31), c0 = 2 * (lane >> 5);
     const v4i lo = *(const v4i*) (st + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + fa_pos(r, c0 + 1) * 16);
     f.a[i] = v8i {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
 
-// B stored n-contiguous: transposed LDS reads
-__device__ __forceinline__ void read_b_tr(Frags& f, int j, const char* st, int wn, int lane)
+// B stored n-contiguous: transposed LDS reads (cb0: the wavefront's first 16-column chunk of the tile)
+template<class FR>
+__device__ __forceinline__ void read_b_tr(FR& f, int j, const char* st, int cb0, int lane)
 {
-    const int q = lane >> 4, cb = wn * 4 + j * 2 + (q & 1), g = q >> 1, rr = (lane & 15) >> 1, h = lane & 1;
+    const int q = lane >> 4, cb = cb0 + j * 2 + (q & 1), g = q >> 1, rr = (lane & 15) >> 1, h = lane & 1;
     v2i       t[4];
 #pragma unroll
     for (int tt = 0; tt < 4; tt++)
@@ -58,10 +62,11 @@ __device__ __forceinline__ void read_b_tr(Frags& f, int j, const char* st, int w
 // row XOR-swizzled by k & 3.  ds_read_b64_tr_b16: within a group of 16 lanes, lane q addresses the 8-byte piece q % 4 of
 // row q / 4 and receives 4 consecutive k of its own column.  The fragment's k order ({0-7, 16-23} then {8-15, 24-31}
 // for the two lane halves) is the one the k-contiguous reads of the other operand produce.
-__device__ __forceinline__ void read_b_tr16(Frags& f, int j, const char* st, int wn, int lane)
+template<class FR>
+__device__ __forceinline__ void read_b_tr16(FR& f, int j, const char* st, int cb0, int lane)
 {
     typedef short v4s __attribute__((ext_vector_type(4)));
-    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wn * 4 + j * 2 + (g & 1);
+    const int g = lane >> 4, q = lane & 15, h = g >> 1, block = cb0 + j * 2 + (g & 1);
     union
     {
         v4s h4[4];
@@ -79,8 +84,8 @@ __device__ __forceinline__ void read_b_tr16(Frags& f, int j, const char* st, int
 
 // bf16, A stored f-contiguous: the same stage layout and reads as an n-contiguous B, over the wavefront's TM / 2 rows
 // (a k-row of the stage is TM elements = TM / 16 blocks of 32 bytes)
-template<int TM>
-__device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int wm, int lane)
+template<int TM, class FR>
+__device__ __forceinline__ void read_a_tr16(FR& f, int i, const char* st, int wm, int lane)
 {
     typedef short v4s __attribute__((ext_vector_type(4)));
     const int g = lane >> 4, q = lane & 15, h = g >> 1, block = wm * (TM / 32) + i * 2 + (g & 1);
@@ -100,7 +105,8 @@ __device__ __forceinline__ void read_a_tr16(Frags& f, int i, const char* st, int
 
 // fp8, A stored f-contiguous: the stage layout and reads of an n-contiguous fp8 B (64 k-rows x 256 bytes), over the
 // wavefront's 128 rows = 8 chunks of 16
-__device__ __forceinline__ void read_a_tr8(Frags& f, int i, const char* st, int wm, int lane)
+template<class FR>
+__device__ __forceinline__ void read_a_tr8(FR& f, int i, const char* st, int wm, int lane)
 {
     const int q = lane >> 4, cb = wm * 8 + i * 2 + (q & 1), g = q >> 1, rr = (lane & 15) >> 1, h = lane & 1;
     v2i       t[4];
@@ -114,9 +120,10 @@ __device__ __forceinline__ void read_a_tr8(Frags& f, int i, const char* st, int 
 }
 
 // B stored k-contiguous (the "abt" form): same layout and reads as A
-__device__ __forceinline__ void read_b_kc(Frags& f, int j, const char* st, int wn, int lane)
+template<class FR>
+__device__ __forceinline__ void read_b_kc(FR& f, int j, const char* st, int cb0, int lane)
 {
-    const int r = wn * 64 + j * 32 + (lane & 31), c0 = 2 * (lane >> 5);
+    const int r = cb0 * 16 + j * 32 + (lane & 31), c0 = 2 * (lane >> 5);
     const v4i lo = *(const v4i*) (st + fa_pos(r, c0) * 16), hi = *(const v4i*) (st + fa_pos(r, c0 + 1) * 16);
     f.b[j] = v8i {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 }
@@ -183,20 +190,29 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[GF_ZERO_PAGE_BYTES
 // NST: stages of the ring (4 to 6, default 4; every instantiation uses the default: six stages of the 128-row tile's 24 KiB
 // measured 2-3 % slower than four on the 3 x 3 convolutions of 32 x 28 x 28 x 256, whose steps then divide by six to find a slot).
 // The reduction has to be at least NST stages long.
-template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST>
+// NW: wavefronts of the workgroup, 8 (2 x 4, each TM / 2 rows x 64 columns, two per SIMD) or 4 (2 x 2, each 128 rows x 128
+// columns with its 256 accumulator registers in the upper half of the 512-register file, one per SIMD: a stage then costs
+// 64 KiB of LDS reads instead of 96; fp8 and AMODE 0 with whole 256-row tiles only).
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST, int NW = 8>
 __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 {
     static_assert(NST >= 4 && NST <= 6 && (!PERSIST || NST == FNST), "ring depth");
+    static_assert(NW == 8 || (NW == 4 && AMODE == 0 && TM == FBM && !RG && !PERSIST && NST == FNST), "four wavefronts: plain k-contiguous A, whole 256-row tiles");
     static_assert(!CHK || (ES == 1 && AMODE == 0 && TM == FBM && !RG), "operand checks: fp8, plain k-contiguous A, whole 256-row tiles");
     static_assert(!PERSIST || (AMODE == 0 && TM == FBM && !RG), "the persistent schedule: plain k-contiguous A, whole 256-row tiles");
     static_assert(TM == 256 || (TM == 128 && AMODE != 2), "the 128-row tile is not instantiated for plain f-contiguous A");
     static_assert(TM == 256 || ES == 2 || AMODE < 2, "fp8 operands that are contiguous along the tile's rows: 256-row tiles only");
     constexpr int  WR = TM / 2;                   // rows per wavefront
     constexpr int  NI = WR / 32;                  // A fragments (32-row blocks) per wavefront
-    constexpr int  NUA = TM / 128;                // A requests per lane and stage (16 rows x 64 bytes per wavefront and request)
+    constexpr int  WGN = NW / 2;                  // the wavefronts form a 2 x WGN grid over the tile
+    constexpr int  WC = FBN / WGN;                // columns per wavefront
+    constexpr int  NJ = WC / 32;                  // B fragments (32-column blocks) per wavefront
+    constexpr int  NUA = TM * FBK / 1024 / NW;    // A requests per lane and stage (16 rows x 64 bytes per wavefront and request)
+    constexpr int  NUB = FBN * FBK / 1024 / NW;   // B requests per lane and stage
     constexpr int  A_BYTES = TM * FBK;            // A part of a stage; the B part follows
     constexpr int  STAGE = A_BYTES + FBK * FBN;   // 32 KiB or 24 KiB
-    constexpr int  NREQ = NUA + 2;                // requests per lane and stage
+    constexpr int  NREQ = NUA + NUB;              // requests per lane and stage
+    using Frags = FragsT<NJ>;
     constexpr bool GATHER = AMODE == 1;           // tap masks + uniform tap offsets
     static_assert(!RG || AMODE != 2, "partial tiles are not instantiated for plain f-contiguous A");
     constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3 || RG; // the last row tile may be partial
@@ -206,7 +222,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     warm_kernargs(g);
     if (!CHK && g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
 
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave >> 2, wn = wave & 3;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), wm = wave / WGN, wn = wave % WGN;
     const int tiles_n = RG ? (g.N + FBN - 1) / FBN : g.N / FBN, tiles_m = (g.M + TM - 1) / TM;
     const int tiles_total = tiles_m * tiles_n;
     int       m0 = 0, n0 = 0, b0 = 0, b1 = 0, b2 = 0, cur_tm = 0, cur_tn = 0;
@@ -270,25 +286,25 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         locate(blockIdx.x, blockIdx.y);
     const uint32_t  lds_base = (uint32_t) (uintptr_t) lds;
 
-    v16f acc[NI][2];
+    v16f acc[NI][NJ];
 #pragma unroll
     for (int i = 0; i < NI; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NJ; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
     // split-k: slice `kslice` takes an equal share of the stages and writes raw partial sums to the workspace
     const int nk = g.K * ES / FBK / (g.split_k > 1 ? g.split_k : 1), kt_begin = kslice * nk;
-    // per-lane global pointers of this wavefront's 2 + 2 request slots (they advance by one stage per step)
-    const uint8_t* ga[2];
-    const uint8_t* gb[2];
+    // per-lane global pointers of this wavefront's request slots (they advance by one stage per step)
+    const uint8_t* ga[NUB];
+    const uint8_t* gb[NUB];
     auto setup_ptrs = [&]() __attribute__((always_inline))
     {
 #pragma unroll
-    for (int u = 0; u < 2; u++)
+    for (int u = 0; u < NUB; u++)
     {
-        const int t = wave * 2 + u;
+        const int t = wave * NUB + u;
         ga[u] = nullptr;
         if constexpr (AMODE == 0)
         {
@@ -329,7 +345,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     };
     setup_ptrs();
     // ---- GATHER: per-row tap masks and the running (tap, channel) position of the stage being requested ----------------
-    uint32_t  tap_ok[2] = {0, 0};      // bit t: tap t of this lane's row (request slot u) reads inside the source tensor
+    uint32_t  tap_ok[NUB] = {};        // bit t: tap t of this lane's row (request slot u) reads inside the source tensor
     int       g_tap = 0, g_ch = 0;     // uniform: tap and first channel of the next stage to request
     int       g_t[3] = {0, 0, 0};      // g_tap as (s, r, q)
     int       g_chb = 0;               // uniform: g_ch in bytes
@@ -337,7 +353,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     long long g_step_b = 0;            // plain weights: bytes from one stage to the next
     // per lane and request slot: where the current tap's channels of this lane's row start, or the zero page when the tap
     // falls into the padding (the zero page is as long as a row's channels, so every lane adds the same channel offset)
-    const uint8_t* a_tap[2] = {nullptr, nullptr};
+    const uint8_t* a_tap[NUB] = {};
     const int stage_ch = FBK / ES;     // channels per stage
     // (values that are the same in every lane are handed back to scalar registers after the vector arithmetic of a tap change)
     auto uniform32 = [](int x) __attribute__((always_inline)) { return __builtin_amdgcn_readfirstlane(x); };
@@ -564,19 +580,20 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         if constexpr (GATHER)
         {
             // one running offset for both kinds of weights, so the step has no branch on the kind
-            dma16(gb[u] + g_delta_b, lds_base + slot * STAGE + A_BYTES + (wave * 2 + u) * 1024);
-            if (u == 1) gather_advance(); // the stage's last request
+            dma16(gb[u] + g_delta_b, lds_base + slot * STAGE + A_BYTES + (wave * NUB + u) * 1024);
+            if (u == NUB - 1) gather_advance(); // the stage's last request
             return;
         }
-        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * STAGE + A_BYTES + (wave * 2 + u) * 1024);
+        dma16(gb[u] + (B_KC ? (size_t) stage * FBK : (size_t) stage * (FBK / ES) * ldb), lds_base + slot * STAGE + A_BYTES + (wave * NUB + u) * 1024);
     };
     auto read_b = [&](Frags & f, int j, const char* st) __attribute__((always_inline))
     {
-        if (B_KC) read_b_kc(f, j, st + A_BYTES, wn, lane);
+        // (the wavefront's first 16-column chunk of the tile)
+        if (B_KC) read_b_kc(f, j, st + A_BYTES, wn * (WC / 16), lane);
         else if (ES == 1)
-            read_b_tr(f, j, st + A_BYTES, wn, lane);
+            read_b_tr(f, j, st + A_BYTES, wn * (WC / 16), lane);
         else
-            read_b_tr16(f, j, st + A_BYTES, wn, lane);
+            read_b_tr16(f, j, st + A_BYTES, wn * (WC / 16), lane);
     };
 
     // all four slots of the ring are requested up front: a slot is free again as soon as its stage has been copied into
@@ -586,7 +603,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         for (int t = 0; t < NST; t++)
         {
 #pragma unroll
-            for (int u = 0; u < 2; u++)
+            for (int u = 0; u < NUB; u++)
             {
                 if (u < NUA) issue_a(u, t, t);
                 issue_b(u, t, t);
@@ -605,7 +622,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #pragma unroll
         for (int i = 0; i < NI; i++)
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < NJ; j++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
     }
@@ -622,7 +639,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #pragma unroll
     for (int i = 0; i < NI; i++) read_a_any(f, i, lds);
 #pragma unroll
-    for (int j = 0; j < 2; j++) read_b(f, j, lds);
+    for (int j = 0; j < NJ; j++) read_b(f, j, lds);
 
     constexpr bool MSCALE = ES == 1 && AMODE == 0 && TM == FBM && !RG && !PERSIST && !CHK;
     const int      mfma_scale_a = 127 + (MSCALE ? g.epi.mfma_scale_exp : 0);
@@ -669,15 +686,20 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     if (LOADS) issue_a(u, t + NST, slot);
 #define LB(u) \
     if (LOADS) issue_b(u, t + NST, slot);
-    // the look itself: this wavefront's eighth (2 KiB) of one operand's part of a stage, straight from LDS (the swizzled
+    // the look itself: this wavefront's share (2 KiB of eight wavefronts, 4 KiB of four) of one operand's part of a stage, straight from LDS (the swizzled
     // placement does not matter, every byte of the part is an operand byte)
     auto chk_scan = [&](const char* part, uint32_t mask, uint32_t add) __attribute__((always_inline))
     {
-        const v4i x0 = *(const v4i*) (part + wave * 2048 + lane * 16), x1 = *(const v4i*) (part + wave * 2048 + 1024 + lane * 16);
-        chk_bad |= (((uint32_t) x0.x & mask) + add) | (((uint32_t) x0.y & mask) + add);
-        chk_bad |= (((uint32_t) x0.z & mask) + add) | (((uint32_t) x0.w & mask) + add);
-        chk_bad |= (((uint32_t) x1.x & mask) + add) | (((uint32_t) x1.y & mask) + add);
-        chk_bad |= (((uint32_t) x1.z & mask) + add) | (((uint32_t) x1.w & mask) + add);
+#pragma unroll
+        for (int q = 0; q < 8 / NW; q++)
+        {
+            const char* mine = part + wave * (16384 / NW) + q * 2048 + lane * 16;
+            const v4i   x0 = *(const v4i*) mine, x1 = *(const v4i*) (mine + 1024);
+            chk_bad |= (((uint32_t) x0.x & mask) + add) | (((uint32_t) x0.y & mask) + add);
+            chk_bad |= (((uint32_t) x0.z & mask) + add) | (((uint32_t) x0.w & mask) + add);
+            chk_bad |= (((uint32_t) x1.x & mask) + add) | (((uint32_t) x1.y & mask) + add);
+            chk_bad |= (((uint32_t) x1.z & mask) + add) | (((uint32_t) x1.w & mask) + add);
+        }
     };
     // steps until this workgroup's next turn to look at the A part / B part of a stage: stage s of the A rows falls to the tile
     // column s mod tiles_n, of the B columns to the tile row s mod tiles_m; step t looks at stage t + 1 (stage 0 right here)
@@ -740,6 +762,29 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             }
         }
         FENCE;
+        if constexpr (NJ == 4)
+        {
+            // one wavefront per SIMD, 16 MFMAs per stage: column by column through rows 0 and 1, then through rows 2 and 3.  A
+            // fragment is refilled right after its last use and then has six or more MFMAs (400 cycles) until its next use in
+            // the following stage; the eight requests ride along in the first half
+            MMA(1, 0); FENCE;
+            LA(0) MMA(0, 1); FENCE;
+            LA(1) MMA(1, 1); FENCE;
+            LA(2) MMA(0, 2); FENCE;
+            LA(3) MMA(1, 2); FENCE;
+            LB(0) MMA(0, 3); FENCE;
+            RA(0) LB(1) MMA(1, 3); FENCE;
+            RA(1) LB(2) MMA(2, 0); FENCE;
+            LB(3) MMA(3, 0); FENCE;
+            RB(0) MMA(2, 1); FENCE;
+            MMA(3, 1); FENCE;
+            RB(1) MMA(2, 2); FENCE;
+            MMA(3, 2); FENCE;
+            RB(2) MMA(2, 3); FENCE;
+            RA(2) MMA(3, 3); FENCE;
+            RB(3) RA(3) FENCE;
+            return;
+        }
         MMA(0, 1); FENCE;
         if constexpr (NI == 4)
         {
@@ -768,7 +813,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     // steps 0 .. nk-NST-1 request stages NST .. nk-1.  The 128-row tile walks the four-stage ring four steps at a time: t is
     // then a multiple of four, the slots of a step are compile-time constants and the LDS addresses of its reads and
     // requests need no arithmetic; what is left of the steps (a pair, the count is even) follows.
-    if constexpr (TM == 128 && NST == 4 && !PERSIST)
+    if constexpr ((TM == 128 || NW == 4) && NST == 4 && !PERSIST)
         for (; t + NST + 3 < nk; t += 4)
         {
             step(t, WM {}, T {}, T {});
@@ -849,7 +894,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         asm volatile("" : "+v"(elane));
         asm volatile("" : "+s"(ewave));
     }
-    const int ewm = ewave >> 2, ewn = ewave & 3;
+    const int ewm = ewave / WGN, ewn = ewave % WGN;
     const long long ldc = g.epi.ld;
     const bool      has_alpha = g.epi.has_alpha != 0;
     const float     alpha = g.epi.alpha;
@@ -861,8 +906,21 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
                            g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
     const int       kg = elane >> 5;
     const bool      finite = g.epi.finite != 0;
-    // element offset of this elane's first value in block (0, 0): row em0 + ewm * WR + elane % 32, column en0 + ewn * 64 + 16 kg
-    const long long lane_elem = c_off + (long long) (em0 + ewm * WR + (elane & 31)) * ldc + en0 + ewn * 64 + kg * 16;
+    // element offset of this elane's first value in block (0, 0): row em0 + ewm * WR + elane % 32, column en0 + ewn * WC + 16 kg
+    const long long lane_elem = c_off + (long long) (em0 + ewm * WR + (elane & 31)) * ldc + en0 + ewn * WC + kg * 16;
+    // (four wavefronts: the 256 accumulators live in the accumulation registers; reading each one from there where it is used
+    // keeps the register allocator from moving them all to vector registers, and from there to scratch memory, at once)
+    auto acc_value = [&](float x) __attribute__((always_inline))
+    {
+        if constexpr (NW == 4)
+        {
+            float y;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(y) : "a"(x));
+            return y;
+        }
+        else
+            return x;
+    };
     // block (i, j) -> the elane's 16 values after the power-of-two factors and relu
     auto gather = [&](int i, int j, float (&val)[16], auto raw_c) __attribute__((always_inline))
     {
@@ -871,7 +929,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #pragma unroll
             for (int r = 0; r < 4; r++)
             {
-                const float lo = acc[i][j][4 * q + r], hi = acc[i][j][8 + 4 * q + r];
+                const float lo = acc_value(acc[i][j][4 * q + r]), hi = acc_value(acc[i][j][8 + 4 * q + r]);
                 const auto  sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
                 val[8 * q + r] = __uint_as_float(sw[0]);
                 val[8 * q + 4 + r] = __uint_as_float(sw[1]);
@@ -885,7 +943,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         if (col_exp)
         {
 #pragma unroll
-            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[RG ? min(en0 + ewn * 64 + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * 64 + j * 32 + kg * 16 + c]);
+            for (int c = 0; c < 16; c++) val[c] *= pow2_of(col_exp[RG ? min(en0 + ewn * WC + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * WC + j * 32 + kg * 16 + c]);
         }
         if (relu)
         {
@@ -899,7 +957,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     typedef __bf16   e_v2bf __attribute__((ext_vector_type(2)));
     // Converted values pass through LDS on their way out (the ring is idle by now): a elane holds 16 columns of one row, and
     // stored from there a 128-byte line of the output would arrive as four to eight separate pieces.  Each wavefront stages
-    // one 32-row block of its 64 columns (16-byte chunks XOR-swizzled by row, conflict-free both ways) and stores it back
+    // one 32-row block of 64 of its columns (16-byte chunks XOR-swizzled by row, conflict-free both ways) and stores it back
     // with consecutive lanes on consecutive chunks of a row: whole lines per request.
     auto walk_to = [&](auto esz_c, auto raw_c, uint8_t* outb, long long pitch, auto pack) __attribute__((always_inline))
     {
@@ -910,15 +968,69 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         const int     row = elane & 31, swz = (row * CPR / 16) & (CPR - 1);
         constexpr bool RAW = decltype(raw_c)::value; // partial sums of a k-slice: no factors, no relu
         if constexpr (!PERSIST) __syncthreads(); // the slowest wavefront has taken its last fragments out of the ring
+        if constexpr (NW == 4)
+        {
+            // One wavefront per SIMD: nothing else covers the two LDS round trips of a block, so the blocks are pipelined by
+            // hand through two staging buffers: while block n comes back from LDS, block n + 1 is converted; while block n's
+            // stores leave, block n + 1 goes into the other buffer.
+            constexpr int NB = NI * (NJ / 2), BUF = NW * 32 * RB;
+            uint32_t      p0[4 * ESZ], p1[4 * ESZ];
+            auto convert = [&](int n) __attribute__((always_inline))
+            {
+                float val[16];
+                gather(n / (NJ / 2), (n % (NJ / 2)) * 2, val, raw_c);
+                pack(val, p0);
+                gather(n / (NJ / 2), (n % (NJ / 2)) * 2 + 1, val, raw_c);
+                pack(val, p1);
+            };
+            auto lds_put = [&](int buf) __attribute__((always_inline))
+            {
+#pragma unroll
+                for (int h = 0; h < ESZ; h++)
+                {
+                    *(e_v4u*) (stg + buf * BUF + row * RB + ((((0 * 2 + kg) * ESZ + h) ^ swz) << 4)) = e_v4u {p0[4 * h], p0[4 * h + 1], p0[4 * h + 2], p0[4 * h + 3]};
+                    *(e_v4u*) (stg + buf * BUF + row * RB + ((((1 * 2 + kg) * ESZ + h) ^ swz) << 4)) = e_v4u {p1[4 * h], p1[4 * h + 1], p1[4 * h + 2], p1[4 * h + 3]};
+                }
+            };
+            convert(0);
+            lds_put(0);
+#pragma unroll
+            for (int n = 0; n < NB; n++)
+            {
+                const int i = n / (NJ / 2), jh = n % (NJ / 2);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                e_v4u v[NRD];
+#pragma unroll
+                for (int r = 0; r < NRD; r++)
+                {
+                    const int q = r * 64 + elane, rr = q / CPR, lc = q % CPR;
+                    v[r] = *(const e_v4u*) (stg + (n & 1) * BUF + rr * RB + ((lc ^ ((rr * CPR / 16) & (CPR - 1))) << 4));
+                }
+                if (n + 1 < NB) convert(n + 1);
+#pragma unroll
+                for (int r = 0; r < NRD; r++)
+                {
+                    const int q = r * 64 + elane, rr = q / CPR, lc = q % CPR;
+                    if ((!RAGGED_M || em0 + ewm * WR + i * 32 + rr < g.M) && (!RG || en0 + ewn * WC + jh * 64 + lc * (16 / ESZ) < g.N))
+                        __builtin_nontemporal_store(v[r], (e_v4u*) (outb + (long long) (i * 32 + rr) * pitch + jh * RB + lc * 16));
+                }
+                if (n + 1 < NB) lds_put((n + 1) & 1);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < NI; i++)
+#pragma unroll
+        for (int jh = 0; jh < NJ / 2; jh++) // (64 columns at a time)
         {
 #pragma unroll
             for (int j = 0; j < 2; j++)
             {
                 float    val[16];
                 uint32_t pk[4 * ESZ];
-                gather(i, j, val, raw_c);
+                gather(i, jh * 2 + j, val, raw_c);
                 pack(val, pk);
 #pragma unroll
                 for (int h = 0; h < ESZ; h++)
@@ -932,8 +1044,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             {
                 const int   q = r * 64 + elane, rr = q / CPR, lc = q % CPR;
                 const e_v4u v = *(const e_v4u*) (stg + rr * RB + ((lc ^ ((rr * CPR / 16) & (CPR - 1))) << 4));
-                if ((!RAGGED_M || em0 + ewm * WR + i * 32 + rr < g.M) && (!RG || en0 + ewn * 64 + lc * (16 / ESZ) < g.N))
-                    __builtin_nontemporal_store(v, (e_v4u*) (outb + (long long) (i * 32 + rr) * pitch + lc * 16));
+                if ((!RAGGED_M || em0 + ewm * WR + i * 32 + rr < g.M) && (!RG || en0 + ewn * WC + jh * 64 + lc * (16 / ESZ) < g.N))
+                    __builtin_nontemporal_store(v, (e_v4u*) (outb + (long long) (i * 32 + rr) * pitch + jh * RB + lc * 16));
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
@@ -943,12 +1055,12 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     auto walk = [&](auto esz_c, auto pack) __attribute__((always_inline))
     {
         constexpr int ESZ = decltype(esz_c)::value;
-        walk_to(esz_c, std::false_type(), (uint8_t*) g.epi.out + (c_off + (long long) (em0 + ewm * WR) * ldc + en0 + ewn * 64) * ESZ, ldc * ESZ, pack);
+        walk_to(esz_c, std::false_type(), (uint8_t*) g.epi.out + (c_off + (long long) (em0 + ewm * WR) * ldc + en0 + ewn * WC) * ESZ, ldc * ESZ, pack);
     };
     if (!PERSIST && g.split_k > 1)
     {
         // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
-        float* ws = g.workspace + ((long long) kslice * gridDim.y + blockIdx.y) * g.M * (long long) g.N + (long long) (em0 + ewm * WR) * g.N + en0 + ewn * 64;
+        float* ws = g.workspace + ((long long) kslice * gridDim.y + blockIdx.y) * g.M * (long long) g.N + (long long) (em0 + ewm * WR) * g.N + en0 + ewn * WC;
         walk_to(std::integral_constant<int, 4>(), std::true_type(), (uint8_t*) ws, (long long) g.N * 4, [&](const float (&val)[16], uint32_t (&pk)[16]) __attribute__((always_inline)) {
 #pragma unroll
             for (int c = 0; c < 16; c++) pk[c] = __float_as_uint(val[c]);
@@ -1032,7 +1144,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #pragma unroll 1
         for (int i = 0; i < NI; i++)
 #pragma unroll 1
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < NJ; j++)
             {
                 float val[16];
 #pragma unroll
@@ -1045,11 +1157,11 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #pragma unroll
                         for (int ii = 0; ii < NI; ii++)
 #pragma unroll
-                            for (int jj = 0; jj < 2; jj++)
+                            for (int jj = 0; jj < NJ; jj++)
                                 if (ii == i && jj == j)
                                 {
-                                    lo = acc[ii][jj][4 * q + r];
-                                    hi = acc[ii][jj][8 + 4 * q + r];
+                                    lo = acc_value(acc[ii][jj][4 * q + r]);
+                                    hi = acc_value(acc[ii][jj][8 + 4 * q + r]);
                                 }
                         const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
                         val[8 * q + r] = __uint_as_float(sw[0]);
@@ -1059,8 +1171,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
                 {
                     float x = val[c];
                     if (has_alpha) x *= alpha;
-                    if (col_exp) x *= pow2_of(col_exp[RG ? min(en0 + ewn * 64 + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * 64 + j * 32 + kg * 16 + c]);
-                    if ((!RAGGED_M || em0 + ewm * WR + i * 32 + (elane & 31) < g.M) && (!RG || en0 + ewn * 64 + j * 32 + kg * 16 < g.N)) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
+                    if (col_exp) x *= pow2_of(col_exp[RG ? min(en0 + ewn * WC + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * WC + j * 32 + kg * 16 + c]);
+                    if ((!RAGGED_M || em0 + ewm * WR + i * 32 + (elane & 31) < g.M) && (!RG || en0 + ewn * WC + j * 32 + kg * 16 < g.N)) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
                 }
             }
     }
@@ -1082,20 +1194,20 @@ __device__ __forceinline__ void clock_probe_stamp(KARG GemmProblem& g, int at_en
     probe[4 * wg + 2 * at_end + 1] = wall_clock64();
 }
 
-template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST>
+template<int ES, int FMT, bool B_KC, int AMODE = 0, int TM = FBM, bool RG = false, bool PERSIST = false, bool CHK = false, int NST = FNST, int NW = 8>
 __device__ __forceinline__ void gemm_fast_body(KARG GemmProblem& g)
 {
     // (a launch that its predicate skips leaves the cells to the launch that ran)
     const bool probe = g.clock_probe && !(!CHK && g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0)));
     if (probe) clock_probe_stamp(g, 0);
-    gemm_fast_body_impl<ES, FMT, B_KC, AMODE, TM, RG, PERSIST, CHK, NST>(g);
+    gemm_fast_body_impl<ES, FMT, B_KC, AMODE, TM, RG, PERSIST, CHK, NST, NW>(g);
     if (probe) clock_probe_stamp(g, 1);
 }
 
 
 // sets the dynamic-LDS limit once per kernel, then launches
 template<class K>
-hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s, int tile_m = FBM, int stages = FNST)
+hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 grid, hipStream_t s, int tile_m = FBM, int stages = FNST, int lanes = 512)
 {
     const int lds_bytes = stages * (tile_m * FBK + FBK * FBN);
     if (!attr_done)
@@ -1104,7 +1216,7 @@ hipError_t launch_fast(K kernel, bool& attr_done, const GemmProblem& p, dim3 gri
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(512), lds_bytes, s, p);
+    hipLaunchKernelGGL(kernel, grid, dim3(lanes), lds_bytes, s, p);
     return hipGetLastError();
 }
 } // namespace

@@ -88,6 +88,7 @@ struct mme_hip_calc
     DeviceBuffer          flag;      // one 32-bit cell: epoch number of the latest call whose operands held codes the hardware formats lack
     uint32_t              specials_epoch = 0; // epoch number of the latest call that scanned
     int                   fp8_specials_policy = 0;
+    int                   last_form[4] = {0, 256, 1, 8}; // mme_hip_last_contraction_form
     // set for the duration of a call through the entry point that allocates nothing: every workspace comes out of the
     // device's static scratch array (noalloc_used: bytes handed out so far in this call)
     bool                  noalloc = false;
@@ -359,6 +360,11 @@ int plan_launch(mme_hip_handle h, GemmProblem& g)
 {
     g.tile_m = gemm_fast_pick_tile_m(g, h->num_cus);
     g.split_k = gemm_pick_split_k(g, h->num_cus);
+    g.waves = gemm_fast_pick_waves(g, h->num_cus);
+    h->last_form[0] = gemm_large_tile_applicable(g) ? 1 : 0;
+    h->last_form[1] = g.tile_m == 128 ? 128 : 256;
+    h->last_form[2] = g.split_k > 1 ? g.split_k : 1;
+    h->last_form[3] = g.waves == 4 ? 4 : 8;
     g.workspace = nullptr;
     g.clock_probe = h->clock_probe;
     if (g.split_k > 1)
@@ -872,6 +878,16 @@ int mme_hip_clock_probe_read(mme_hip_handle h, double* shader_mhz, double* mean_
     if (shader_mhz) *shader_mhz = n ? clocks / ticks * 100.0 : 0.0;
     if (mean_us) *mean_us = n ? ticks / n / 100.0 : 0.0;
     if (max_us) *max_us = worst / 100.0;
+    return MME_HIP_OK;
+}
+
+int mme_hip_last_contraction_form(mme_hip_handle h, int* large_tile, int* tile_rows, int* split_k, int* wavefronts)
+{
+    if (!h) return MME_HIP_EINVAL;
+    if (large_tile) *large_tile = h->last_form[0];
+    if (tile_rows) *tile_rows = h->last_form[1];
+    if (split_k) *split_k = h->last_form[2];
+    if (wavefronts) *wavefronts = h->last_form[3];
     return MME_HIP_OK;
 }
 

@@ -124,6 +124,7 @@ struct GemmProblem
     OperandView  A, B;
     GemmEpilogue epi;
     int          tile_m;     // large-tile kernel: rows of the output tile, 128 or 0 / 256 (chosen by gemm_fast_pick_tile_m)
+    int          waves;      // large-tile kernel: wavefronts per workgroup, 4 or 0 / 8 (chosen by gemm_fast_pick_waves)
     int          split_k;    // >1: partial sums go to workspace and are reduced in a fixed order
     float*       workspace;  // split_k * batch * M * N floats
     // device-side predicate: when skip_flag != NULL the whole launch returns at once if (*skip_flag == skip_epoch) == skip_if
@@ -160,6 +161,7 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s);
 // large aligned fp8 problems (gemm_large_tile.hip); launch_gemm routes to it when applicable
 bool       gemm_large_tile_applicable(const GemmProblem& p);
 int        gemm_fast_pick_split_k(const GemmProblem& p, int num_cus); // 0: the large-tile kernel does not take this problem
+int        gemm_fast_pick_waves(const GemmProblem& p, int num_cus);   // (after tile_m and split_k have been chosen)
 hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s);
 // the kernel this problem takes can check its fp8 operands for special codes itself (GemmProblem::chk)
 bool       gemm_large_tile_checks_operands(const GemmProblem& p);

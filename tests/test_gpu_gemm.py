@@ -202,6 +202,70 @@ def test_fp8_special_codes_found_by_the_large_tile_kernel(calc, orc, M, N, K, dt
     assert np.isfinite(got).all() and rel_frobenius(got[:16].ravel(), expected(want)) <= tol
 
 
+@pytest.mark.parametrize("policy", [abi.FP8_SPECIALS_CHECK, abi.FP8_SPECIALS_ASSUME_NONE])
+@pytest.mark.parametrize("M,N,K,op,dtA,bA,dtB,bB,out_dt", [
+    (4096, 4096, 3072, abi.OP_AB, abi.FP8_143, 7, abi.FP8_143, 7, abi.BF16), (4096, 4096, 3072, abi.OP_ABT, abi.FP8_143, 11, abi.FP8_152, 15, abi.FP32),
+    (3072, 4096, 4096, abi.OP_AB, abi.FP8_152, 15, abi.FP8_143, 3, abi.FP8_143), (3072, 4096, 4096, abi.OP_ABT, abi.FP8_152, 17, abi.FP8_152, 12, abi.BF16)])
+def test_fp8_four_wavefront_form_vs_oracle(calc, orc, policy, M, N, K, op, dtA, bA, dtB, bB, out_dt):
+    """One round of tiles and a long reduction: the fp8 GEMM runs in its form with four wavefronts of 128 x 128 outputs per
+    workgroup (4096 x 4096 outputs = 256 workgroups of 48 stages; 3072 x 4096 outputs = 192 workgroups of 64 stages; with
+    half as many tiles or fewer the 128-row tiles take over, so this form never meets split-k).  Both operand policies (with and without the
+    in-kernel look at the operand bytes), every fp8 flavour pair, B stored either way, raw fp32 and fused bf16 / fp8
+    outputs: 16-row slabs from four tile rows (tile boundaries included) plus 32 random rows against the oracle, every
+    column; the fused outputs also bit for bit against the oracle's cast of the GPU's own fp32 accumulators."""
+    import torch
+    rng = np.random.default_rng(77 + op + dtA)
+    asz, bsz = _shapes(op, M, N, K)
+    a = random_operand(rng, dtA, M * K, orc, bA, 0)
+    b = random_operand(rng, dtB, K * N, orc, bB, 0)
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    acc_gpu = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    X, Wt = MmeSimTensor(asz, 2, dtA, ta, bA), MmeSimTensor(bsz, 2, dtB, tb, bB)
+    calc.setFp8SpecialsPolicy(policy)
+    try:
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, acc_gpu), X, Wt, op)
+        form = calc.lastContractionForm()
+        assert form["large_tile"] and form["tile_rows"] == 256 and form["wavefronts"] == 4, form
+        assert form["split_k"] == 1, form
+        fused = None
+        if out_dt != abi.FP32:
+            fused = torch.zeros(M * N, dtype=torch.int16 if out_dt == abi.BF16 else torch.uint8, device="cuda")
+            calc.doBatchGemm(MmeSimTensor([N, M], 2, out_dt, fused, 7 if out_dt == abi.FP8_143 else 0), X, Wt, op,
+                             epilogue=Epilogue(scale_exp=-3, clipFp=True))
+            assert calc.lastContractionForm() == form
+        calc.synchronize()
+    finally:
+        calc.setFp8SpecialsPolicy(abi.FP8_SPECIALS_CHECK)
+    got = acc_gpu.cpu().numpy().reshape(M, N)
+    rows = np.concatenate([np.arange(0, 16), np.arange(3 * 256 + 120, 3 * 256 + 136), np.arange(5 * 256 - 8, 5 * 256 + 8), np.arange(M - 16, M),
+                           np.sort(np.random.default_rng(3).choice(M, 32, replace=False))])
+    slab = np.ascontiguousarray(a.reshape(M, K)[rows].ravel())
+    want = np.zeros(rows.size * N, np.float32)
+    assert orc.orc_batch_gemm(A(desc(want, [N, rows.size], abi.FP32)), A(desc(slab, [K, rows.size], dtA, bA)), A(desc(b, bsz, dtB, bB)), op) == 0
+    dist = rel_frobenius(got[rows].ravel(), want)
+    assert dist <= 1e-2
+    assert dist <= 1e-4  # the reference's truncating tree itself sits ~1e-5 from the exact sums
+    assert np.count_nonzero(got.reshape(M // 256, 256, N // 256, 256), axis=(1, 3)).min() > 256 * 256 // 2  # every tile was written
+    if fused is not None:
+        codes = np.zeros(M * N, np.uint16 if out_dt == abi.BF16 else np.uint8)
+        flat = np.ascontiguousarray(got.ravel())
+        assert orc.orc_cast_from_fp32(codes.ctypes.data, out_dt, 7 if out_dt == abi.FP8_143 else 0, 0, flat.ctypes.data, M * N, -3, None, 0, 0, 0, 1, 0, 0) == 0
+        assert np.array_equal(fused.cpu().numpy().view(codes.dtype), codes)
+
+
+def test_fp8_short_reductions_keep_eight_wavefronts(calc):
+    """Below 48 stages per workgroup, or with more tiles than one round, the form with eight wavefronts stays."""
+    import torch
+    for M, N, K, waves in ((4096, 4096, 1024, 8), (4096, 4096, 4096, 4), (8192, 8192, 4096, 8), (512, 512, 512, 8)):
+        ta, tb = torch.zeros(M * K, dtype=torch.uint8, device="cuda"), torch.zeros(K * N, dtype=torch.uint8, device="cuda")
+        out = torch.zeros(M * N, dtype=torch.int16, device="cuda")
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.BF16, out), MmeSimTensor([K, M], 2, abi.FP8_143, ta, 7), MmeSimTensor([N, K], 2, abi.FP8_143, tb, 7),
+                         abi.OP_AB, epilogue=Epilogue(scale_exp=-2, clipFp=True))
+        calc.synchronize()
+        form = calc.lastContractionForm()
+        assert form["large_tile"] and form["wavefronts"] == waves, (M, N, K, form)
+
+
 def test_fp8_special_codes_take_exact_path(calc, orc):
     """fp8_143 in full inf/nan mode: exponent-15 codes are inf / NaN for Gaudi and finite for the hardware's e4m3.
     The library must notice them and still agree with the reference (NaN / inf placement included)."""
