@@ -78,7 +78,8 @@ class Bench:
         """Calls fn back to back for some tens of milliseconds.  After an idle period (operand set-up on the host) the device
         needs about 50 ms of work to reach the rate it then sustains: the headline GEMM takes 63-74 us per call over the first
         25 ms, 61 us up to 45 ms, and 59.7-59.9 us from there on for as long as it was watched (2.5 s).  Every measurement here
-        is of the sustained rate, so each one starts from a device that is already at work."""
+        is of the sustained rate, so each one starts from a device that is already at work (0.06, 0.5 and 2 s of it give the
+        same figures for the GEMMs and the convolutions)."""
         t0 = time.perf_counter()
         while time.perf_counter() - t0 < seconds:
             for _ in range(10):
@@ -102,15 +103,22 @@ class Bench:
 
     def clocked(self, fn, n=30):
         """The shader clock the large-tile kernels ran at during n back-to-back calls of fn, and how long a workgroup took
-        (stamps taken inside the kernels; the published peak rates are quoted at 2400 MHz)."""
+        (stamps taken inside the kernels; the published peak rates are quoted at 2400 MHz).  call_us_with_probe is the wall
+        time per call while the stamps are on: the probe is not free for every kernel (the persistent walk of the batched
+        GEMM runs 15-20 % slower with it, the one-tile-per-workgroup kernels are not affected), so a clock read here belongs to
+        that time, not to the timed region's."""
         self.calc.clockProbe(True)
+        self.settle(fn)
         self.calc.readClockProbe()
+        t0 = time.perf_counter()
         for _ in range(n):
             fn()
-        r = self.calc.readClockProbe()
+        r = self.calc.readClockProbe()   # (synchronises)
+        wall = time.perf_counter() - t0
         self.calc.clockProbe(False)
         return {"shader_clock_mhz": round(r["shader_mhz"]), "workgroup_us_mean": round(r["workgroup_us_mean"], 2),
-                "workgroup_us_max": round(r["workgroup_us_max"], 2), "workgroups_seen": r["workgroups"]}
+                "workgroup_us_max": round(r["workgroup_us_max"], 2), "workgroups_seen": r["workgroups"],
+                "call_us_with_probe": round(wall / n * 1e6, 2)}
 
     def matrix_core_ceiling(self, dtype):
         """What back-to-back matrix instructions with operands in registers sustain on this device: with all-zero operands
