@@ -104,9 +104,9 @@ class Bench:
     def clocked(self, fn, n=30):
         """The shader clock the large-tile kernels ran at during n back-to-back calls of fn, and how long a workgroup took
         (stamps taken inside the kernels; the published peak rates are quoted at 2400 MHz).  call_us_with_probe is the wall
-        time per call while the stamps are on: the probe is not free for every kernel (the persistent walk of the batched
-        GEMM runs 15-20 % slower with it, the one-tile-per-workgroup kernels are not affected), so a clock read here belongs to
-        that time, not to the timed region's."""
+        time per call while the stamps are on, the read-out of the stamps at the end included (2 us per call at n = 50): the
+        probe is not free for every kernel (the persistent walk of the batched GEMM ran 3 to 17 % slower with it on
+        different boxes), so a clock read here belongs to that time, not to the timed region's."""
         self.calc.clockProbe(True)
         self.settle(fn)
         self.calc.readClockProbe()
@@ -262,7 +262,7 @@ def run_c2(b):
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["fp8"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS["fp8"], 4), "traffic": GEMM_TRAFFIC_BYTES,
                      "kernel": "gemm_fp8_w4_kernel<0, false, true>", "kernel_ms": round(kernel_ms, 5),
-                     "policy": "check (default): the kernel inspects the operand bytes it multiplies; two predicated fall-back launches follow it",
+                     "policy": "check (default): the workgroups inspect the operand bytes they multiply and share what they find per operand panel; a tile whose panels hold a special code is computed again, exactly, inside the same launch",
                      "assume_none": {"achieved": round(assumed, 2), "frac": round(assumed / PEAK_TFLOPS["fp8"], 4), "kernel_ms": round(assumed_s * 1e3, 5),
                                      "kernel": "gemm_fp8_w4_kernel<0, false, false>",
                                      "policy": "the caller promises operands without exponent-all-ones codes (they come out of the saturating quantiser)"}},

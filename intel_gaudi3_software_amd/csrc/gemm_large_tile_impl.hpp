@@ -218,6 +218,12 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3 || RG; // the last row tile may be partial
     // (RG: the last column tile may be partial too; N is a multiple of 16, so a lane's 16 columns are all in or all out)
     constexpr bool A_KC = AMODE < 2;
+    // CHK with four wavefronts (one round of tiles, every workgroup resident): the workgroups take turns at looking like the
+    // eight-wavefront forms do, but note per operand panel what they found and how many of a panel's lookers are done; after its
+    // epilogue a workgroup waits for the lookers of its own two panels (long done by then) and, if one of them met such a code,
+    // computes its tile once more, exactly, inside the same launch (below, after the loop).  No flag for the host, nothing
+    // enqueued behind the kernel.
+    constexpr bool SELFCHK = CHK && NW == 4;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     warm_kernargs(g);
     if (!CHK && g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
@@ -688,7 +694,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     if (LOADS) issue_b(u, t + NST, slot);
     // the look itself: this wavefront's share (2 KiB of eight wavefronts, 4 KiB of four) of one operand's part of a stage, straight from LDS (the swizzled
     // placement does not matter, every byte of the part is an operand byte)
-    auto chk_scan = [&](const char* part, uint32_t mask, uint32_t add) __attribute__((always_inline))
+    uint32_t chk_bad_b = 0; // SELFCHK keeps what it found in B apart from what it found in A (chk_bad)
+    auto chk_scan = [&](const char* part, uint32_t mask, uint32_t add, uint32_t& chk_bad) __attribute__((always_inline))
     {
 #pragma unroll
         for (int q = 0; q < 8 / NW; q++)
@@ -714,8 +721,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         asm volatile("" : "+s"(chk_ma), "+s"(chk_aa), "+s"(chk_mb), "+s"(chk_ab));
         chk_a_mine = chk_ma != 0;
         chk_b_mine = chk_mb != 0;
-        if (cur_tn == 0 && chk_a_mine) chk_scan(lds, chk_ma, chk_aa);
-        if (cur_tm == 0 && chk_b_mine) chk_scan(lds + A_BYTES, chk_mb, chk_ab);
+        if (cur_tn == 0 && chk_a_mine) chk_scan(lds, chk_ma, chk_aa, chk_bad);
+        if (cur_tm == 0 && chk_b_mine) chk_scan(lds + A_BYTES, chk_mb, chk_ab, SELFCHK ? chk_bad_b : chk_bad);
     }
     // One stage: 8 MFMAs; after the first one wait until stage t+1 has landed in every wavefront's view (WAITC leaves the
     // younger stages in flight); each fragment register is refilled from stage t+1 right after its last use in stage t (the
@@ -756,8 +763,8 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
                 chk_cb = chk_cb == 0 ? tiles_m - 1 : chk_cb - 1;
                 if (__builtin_expect(do_a || do_b, 0))
                 {
-                    if (do_a) chk_scan(st, chk_ma, chk_aa);
-                    if (do_b) chk_scan(st + A_BYTES, chk_mb, chk_ab);
+                    if (do_a) chk_scan(st, chk_ma, chk_aa, chk_bad);
+                    if (do_b) chk_scan(st + A_BYTES, chk_mb, chk_ab, SELFCHK ? chk_bad_b : chk_bad);
                 }
             }
         }
@@ -859,11 +866,115 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #undef RB
 #undef LA
 #undef LB
-    if constexpr (CHK)
+    if constexpr (CHK && !SELFCHK)
     {
         if (chk_bad & 0x80808080u) *const_cast<uint32_t*>((const uint32_t*) g.skip_flag) = g.skip_epoch;
         chk_bad = 0;
     }
+    // SELFCHK: what this workgroup's looks found goes into the launch's panel words (GemmProblem::chk_state, zero before the
+    // launch; per batch element: a flag per row panel of A, a flag per column panel of B, then a count of finished lookers
+    // for each), the flags before the counts, all with device scope.
+    bool      tile_exact = false;
+    uint32_t* panel_flag_a = nullptr;
+    uint32_t* panel_flag_b = nullptr;
+    uint32_t* panel_done_a = nullptr;
+    uint32_t* panel_done_b = nullptr;
+    if constexpr (SELFCHK)
+    {
+        uint32_t* st = g.chk_state + (size_t) blockIdx.y * 2u * (unsigned) (tiles_m + tiles_n);
+        panel_flag_a = st + cur_tm;
+        panel_flag_b = st + tiles_m + cur_tn;
+        panel_done_a = st + tiles_m + tiles_n + cur_tm;
+        panel_done_b = st + 2 * tiles_m + tiles_n + cur_tn;
+        const bool bad_a = __syncthreads_or((chk_bad & 0x80808080u) != 0u) != 0, bad_b = __syncthreads_or((chk_bad_b & 0x80808080u) != 0u) != 0;
+        chk_bad = 0;
+        if (threadIdx.x == 0)
+        {
+            // (relaxed device-scope accesses, ordered by hand: the flags are the only data that pass between workgroups, so there
+            // is nothing for a release to write back and nothing for an acquire to invalidate -- with release / acquire every
+            // workgroup flushed and invalidated its L2, 2 us per launch; the wait lets the flag stores be acknowledged before the
+            // counts go out)
+            if (bad_a) __hip_atomic_store(panel_flag_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (bad_b) __hip_atomic_store(panel_flag_b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (bad_a || bad_b) __builtin_amdgcn_s_waitcnt(vm_wait(0));
+            __hip_atomic_fetch_add(panel_done_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(panel_done_b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // The tile once more, from operands decoded to bf16 with Gaudi's meaning of the codes (every fp8 value is a bf16 value;
+    // decoded with the hardware formats' exponent bias, so the epilogue's factor applies unchanged): fragments straight from
+    // global memory, 16 k at a time, v_mfma_f32_32x32x16_bf16 into the same accumulators.  Rare and slow by design (about a
+    // millisecond for K = 4096).
+    auto recompute_exactly = [&]() __attribute__((always_inline))
+    {
+        if constexpr (SELFCHK)
+        {
+            const int mode_a = g.chk_inf_nan_a, mode_b = g.chk_inf_nan_b;
+            // eight codes (two registers) -> eight bf16 (four registers)
+            auto decode8 = [&](uint32_t lo, uint32_t hi, auto e5m2, int mode) __attribute__((always_inline))
+            {
+                uint32_t h[8];
+#pragma unroll
+                for (int q = 0; q < 8; q++)
+                {
+                    const uint32_t code = ((q < 4 ? lo : hi) >> (8 * (q & 3))) & 0xFFu;
+                    h[q] = (decltype(e5m2)::value ? fp8_to_fp32<2>(code, 15, mode) : fp8_to_fp32<3>(code, 7, mode)) >> 16;
+                }
+                union
+                {
+                    uint32_t w[4];
+                    v8bf     v;
+                } u;
+#pragma unroll
+                for (int q = 0; q < 4; q++) u.w[q] = h[2 * q] | (h[2 * q + 1] << 16);
+                return u.v;
+            };
+#pragma unroll
+            for (int i = 0; i < NI; i++)
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+            const int kh = 8 * (lane >> 5), r32 = lane & 31;
+#pragma unroll 1
+            for (int k0 = 0; k0 < g.K; k0 += 16)
+            {
+                v8bf fa[NI], fb[NJ];
+#pragma unroll
+                for (int i = 0; i < NI; i++)
+                {
+                    const uint2 raw = *(const uint2*) (A + (size_t) (m0 + wm * WR + i * 32 + r32) * lda + k0 + kh);
+                    fa[i] = decode8(raw.x, raw.y, std::integral_constant<bool, (FMT & 1) != 0>(), mode_a);
+                }
+#pragma unroll
+                for (int j = 0; j < NJ; j++)
+                {
+                    uint32_t lo = 0, hi = 0;
+                    if constexpr (B_KC)
+                    {
+                        const uint2 raw = *(const uint2*) (B + (size_t) (n0 + wn * WC + j * 32 + r32) * ldb + k0 + kh);
+                        lo = raw.x;
+                        hi = raw.y;
+                    }
+                    else
+                    {
+                        const uint8_t* col = B + (size_t) (k0 + kh) * ldb + n0 + wn * WC + j * 32 + r32;
+#pragma unroll
+                        for (int q = 0; q < 4; q++)
+                        {
+                            lo |= (uint32_t) col[(size_t) q * ldb] << (8 * q);
+                            hi |= (uint32_t) col[(size_t) (q + 4) * ldb] << (8 * q);
+                        }
+                    }
+                    fb[j] = decode8(lo, hi, std::integral_constant<bool, ((FMT >> 1) & 1) != 0>(), mode_b);
+                }
+#pragma unroll
+                for (int i = 0; i < NI; i++)
+#pragma unroll
+                    for (int j = 0; j < NJ; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+            }
+        }
+    };
 
     // ---- epilogue: alpha, per-column power of two, relu, cast, store (same conversion functions as the general kernel).
     // The matrix-core operands are swapped (B fragment first), so accumulator register v of lane l is output column
@@ -905,7 +1016,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     const CastParams cp = {g.epi.cast.dtype,       g.epi.cast.exp_bias, g.epi.cast.inf_nan_mode, g.epi.cast.rm,    g.epi.cast.clip_fp,
                            g.epi.cast.clip_inf_in, g.epi.cast.ftz,      g.epi.cast.relu,         g.epi.cast.scale, g.epi.cast.has_scale};
     const int       kg = elane >> 5;
-    const bool      finite = g.epi.finite != 0;
+    const bool      finite = g.epi.finite != 0; // (SELFCHK: a tile computed again from the decoded operands, which may hold inf and NaN, goes out through the generic converter)
     // element offset of this elane's first value in block (0, 0): row em0 + ewm * WR + elane % 32, column en0 + ewn * WC + 16 kg
     const long long lane_elem = c_off + (long long) (em0 + ewm * WR + (elane & 31)) * ldc + en0 + ewn * WC + kg * 16;
     // (four wavefronts: the 256 accumulators live in the accumulation registers; reading each one from there where it is used
@@ -1057,6 +1168,45 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         constexpr int ESZ = decltype(esz_c)::value;
         walk_to(esz_c, std::false_type(), (uint8_t*) g.epi.out + (c_off + (long long) (em0 + ewm * WR) * ldc + en0 + ewn * WC) * ESZ, ldc * ESZ, pack);
     };
+    // element-wise through the out-of-line generic converter (which applies relu itself): rare cast settings, and the tiles
+    // that the four-wavefront checking form computed again
+    auto store_generic = [&]() __attribute__((always_inline))
+    {
+#pragma unroll 1
+        for (int i = 0; i < NI; i++)
+#pragma unroll 1
+            for (int j = 0; j < NJ; j++)
+            {
+                float val[16];
+#pragma unroll
+                for (int q = 0; q < 2; q++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                    {
+                        // (dynamic block index: read the accumulators through a switch-free copy)
+                        float lo = 0.0f, hi = 0.0f;
+#pragma unroll
+                        for (int ii = 0; ii < NI; ii++)
+#pragma unroll
+                            for (int jj = 0; jj < NJ; jj++)
+                                if (ii == i && jj == j)
+                                {
+                                    lo = acc_value(acc[ii][jj][4 * q + r]);
+                                    hi = acc_value(acc[ii][jj][8 + 4 * q + r]);
+                                }
+                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                        val[8 * q + r] = __uint_as_float(sw[0]);
+                        val[8 * q + 4 + r] = __uint_as_float(sw[1]);
+                    }
+                for (int c = 0; c < 16; c++)
+                {
+                    float x = val[c];
+                    if (has_alpha) x *= alpha;
+                    if (col_exp) x *= pow2_of(col_exp[RG ? min(en0 + ewn * WC + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * WC + j * 32 + kg * 16 + c]);
+                    if ((!RAGGED_M || em0 + ewm * WR + i * 32 + (elane & 31) < g.M) && (!RG || en0 + ewn * WC + j * 32 + kg * 16 < g.N)) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
+                }
+            }
+    };
     if (!PERSIST && g.split_k > 1)
     {
         // raw partial sums; splitk_reduce_kernel adds the slices in order and applies the epilogue
@@ -1139,44 +1289,34 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             fp8_store(std::integral_constant<int, 2>());
     }
     else if (!PERSIST)
+        store_generic();
+    if constexpr (SELFCHK)
     {
-        // rare cast settings: element-wise through the out-of-line generic converter (which applies relu itself)
-#pragma unroll 1
-        for (int i = 0; i < NI; i++)
-#pragma unroll 1
-            for (int j = 0; j < NJ; j++)
+        // every looker of this tile's row panel of A (one workgroup per tile column) and of its column panel of B has finished
+        // its loop before it started the epilogue that this workgroup has just finished as well, so the wait is a formality
+        // unless the device is shared; it is bounded, and a workgroup that cannot tell computes its tile again to be safe
+        bool again = false;
+        if (threadIdx.x == 0)
+        {
+            bool all_in = false;
+            for (int polls = 0; polls < (1 << 14) && !all_in; polls++)
             {
-                float val[16];
-#pragma unroll
-                for (int q = 0; q < 2; q++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                    {
-                        // (dynamic block index: read the accumulators through a switch-free copy)
-                        float lo = 0.0f, hi = 0.0f;
-#pragma unroll
-                        for (int ii = 0; ii < NI; ii++)
-#pragma unroll
-                            for (int jj = 0; jj < NJ; jj++)
-                                if (ii == i && jj == j)
-                                {
-                                    lo = acc_value(acc[ii][jj][4 * q + r]);
-                                    hi = acc_value(acc[ii][jj][8 + 4 * q + r]);
-                                }
-                        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
-                        val[8 * q + r] = __uint_as_float(sw[0]);
-                        val[8 * q + 4 + r] = __uint_as_float(sw[1]);
-                    }
-                for (int c = 0; c < 16; c++)
-                {
-                    float x = val[c];
-                    if (has_alpha) x *= alpha;
-                    if (col_exp) x *= pow2_of(col_exp[RG ? min(en0 + ewn * WC + j * 32 + kg * 16 + c, g.N - 1) : en0 + ewn * WC + j * 32 + kg * 16 + c]);
-                    if ((!RAGGED_M || em0 + ewm * WR + i * 32 + (elane & 31) < g.M) && (!RG || en0 + ewn * WC + j * 32 + kg * 16 < g.N)) store_out_slow(g.epi, lane_elem + (long long) (i * 32) * ldc + j * 32 + c, x);
-                }
+                all_in = __hip_atomic_load(panel_done_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t) tiles_n &&
+                         __hip_atomic_load(panel_done_b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t) tiles_m;
+                if (!all_in) __builtin_amdgcn_s_sleep(16);
             }
+            again = !all_in || __hip_atomic_load(panel_flag_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u ||
+                    __hip_atomic_load(panel_flag_b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+        }
+        if (__builtin_expect(__syncthreads_or(again) != 0, 0))
+        {
+            recompute_exactly();
+            tile_exact = true;
+            store_generic(); // (writes the whole tile again)
+        }
     }
     (void) esz;
+    (void) tile_exact;
     if (!PERSIST || !has_next) break;
     } // walk over tiles
 }

@@ -89,6 +89,10 @@ struct mme_hip_calc
     uint32_t              specials_epoch = 0; // epoch number of the latest call that scanned
     int                   fp8_specials_policy = 0;
     int                   last_form[4] = {0, 256, 1, 8}; // mme_hip_last_contraction_form
+    // panel words of the four-wavefront checking GEMM (GemmProblem::chk_state): a ring of regions, one per launch, all cleared by
+    // one fill launch every CHK_STATE_RING launches
+    DeviceBuffer          chk_state;
+    unsigned              chk_state_launches = 0;
     // set for the duration of a call through the entry point that allocates nothing: every workspace comes out of the
     // device's static scratch array (noalloc_used: bytes handed out so far in this call)
     bool                  noalloc = false;
@@ -127,6 +131,11 @@ int hip_fail(mme_hip_handle h, hipError_t e, const char* what)
 
 // Work space of `bytes` for the current call: the handle's grow-only buffer `buf`, or, in a call that may not allocate, the
 // next piece of the device's static scratch array.
+// panel words of the four-wavefront checking GEMM: words per launch (2 x (row panels + column panels) per batch element, at
+// most 256 tiles in all) and launches per clearing
+constexpr size_t   CHK_STATE_REGION_WORDS = 2048;
+constexpr unsigned CHK_STATE_RING = 64;
+
 int take_ws(mme_hip_handle h, DeviceBuffer& buf, size_t bytes, void** out)
 {
     if (!h->noalloc)
@@ -571,6 +580,45 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         HIP_TRY(h, launch_gemm(g, h->stream));
         return MME_HIP_OK;
     }
+    // the constants of the in-kernel look: a byte b is special when (b & m) == m, m = the exponent field (kind 0) or all of 0x7F
+    // (kind 1: only 0x7F / 0xFF).  An operand in its hardware-native mode is looked at as well, for its inf / NaN codes: the
+    // exact fall-back converts those values like any other, and the native kernel's epilogue may count on finite accumulators.
+    auto set_check_constants = [&]()
+    {
+        const mme_hip_tensor* t[2] = {ta, tb};
+        uint32_t              mask[2], add[2];
+        for (int i = 0; i < 2; i++)
+        {
+            const int      kind = plan.scan_kind[i] >= 0 ? plan.scan_kind[i] : plan.nonfinite_kind[i];
+            const uint32_t m = kind < 0 ? 0u : (kind == 1 ? 0x7Fu : (t[i]->dtype == MME_HIP_FP8_143 ? 0x78u : 0x7Cu));
+            mask[i] = m * 0x01010101u;
+            add[i] = m ? (0x80u - m) * 0x01010101u : 0u;
+        }
+        g.chk_mask_a = mask[0], g.chk_add_a = add[0], g.chk_mask_b = mask[1], g.chk_add_b = add[1];
+        g.chk_inf_nan_a = ta->inf_nan_mode, g.chk_inf_nan_b = tb->inf_nan_mode;
+    };
+    if (in_kernel_check && g.waves == 4)
+    {
+        // the four-wavefront form settles the matter inside its launch (panel words, see GemmProblem::chk_state); it needs
+        // those words, which the allocation-free entry point does not have: that one takes the eight-wavefront form
+        const size_t words = (size_t) g.batch[0] * g.batch[1] * g.batch[2] * 2u * (size_t) (g.M / 256 + g.N / 256);
+        if (h->noalloc || words > CHK_STATE_REGION_WORDS)
+        {
+            g.waves = 8;
+            h->last_form[3] = 8;
+        }
+        else
+        {
+            if (!h->chk_state.p) HIP_TRY(h, h->chk_state.reserve((size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS * sizeof(uint32_t)));
+            const unsigned slot = h->chk_state_launches++ % CHK_STATE_RING;
+            if (slot == 0) HIP_TRY(h, launch_fill_u32((uint32_t*) h->chk_state.p, 0u, (size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS, h->stream));
+            g.chk = 2;
+            g.chk_state = (uint32_t*) h->chk_state.p + (size_t) slot * CHK_STATE_REGION_WORDS;
+            set_check_constants();
+            HIP_TRY(h, launch_gemm(g, h->stream));
+            return MME_HIP_OK;
+        }
+    }
     // the flag holds the epoch of the latest call that met such a code; the native kernel either finds them itself while it
     // multiplies (the large-tile kernels that can) or is skipped when a scan launch in front of it found one; decode + bf16
     // kernel run only when the flag holds this call's epoch, and then write the whole output
@@ -583,20 +631,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     if (in_kernel_check)
     {
         g.chk = 1;
-        const mme_hip_tensor* t[2] = {ta, tb};
-        uint32_t              mask[2], add[2];
-        for (int i = 0; i < 2; i++)
-        {
-            // a byte b is special when (b & m) == m: m = the exponent field (kind 0) or all of 0x7F (kind 1: only 0x7F / 0xFF).
-            // An operand in its hardware-native mode is looked at as well, for its inf / NaN codes: the exact fall-back
-            // converts those values like any other, and the native kernel's epilogue may count on finite accumulators.
-            const int      kind = plan.scan_kind[i] >= 0 ? plan.scan_kind[i] : plan.nonfinite_kind[i];
-            const uint32_t m = kind < 0 ? 0u : (kind == 1 ? 0x7Fu : (t[i]->dtype == MME_HIP_FP8_143 ? 0x78u : 0x7Cu));
-            mask[i] = m * 0x01010101u;
-            add[i] = m ? (0x80u - m) * 0x01010101u : 0u;
-        }
-        g.chk_mask_a = mask[0], g.chk_add_a = add[0], g.chk_mask_b = mask[1], g.chk_add_b = add[1];
-
+        set_check_constants();
     }
     else
         HIP_TRY(h, launch_fp8_special_scan2(flag, epoch, a_base, span_elements(ta), ta->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[0], b_base,
@@ -823,6 +858,7 @@ int mme_hip_set_stream(mme_hip_handle h, void* s)
 {
     if (!h) return MME_HIP_EINVAL;
     h->stream = s ? (hipStream_t) s : h->own_stream;
+    h->chk_state_launches = 0; // (the panel words are cleared in stream order: start a fresh ring on the new stream)
     return MME_HIP_OK;
 }
 

@@ -139,6 +139,13 @@ struct GemmProblem
     // (mask 0: that operand needs no check).  The caller then enqueues the exact fall-back behind it, predicated on the flag.
     int             chk;
     uint32_t        chk_mask_a, chk_add_a, chk_mask_b, chk_add_b; // the byte constants replicated over a 32-bit word
+    // The four-wavefront form (chk == 2; one round of tiles, every workgroup resident) settles the matter inside the launch: the
+    // looks are shared out the same way, but what they find is noted per operand panel in chk_state (zero before the launch,
+    // 2 x (row panels + column panels) words per batch element: flags, then counts of finished lookers), and a workgroup
+    // whose panels hold such a code computes its tile once more, exactly, from operands decoded with Gaudi's meaning of the
+    // codes (inf / NaN modes below; the hardware formats' exponent bias, so that the epilogue's factor stays the same).
+    int             chk_inf_nan_a, chk_inf_nan_b;
+    uint32_t*       chk_state;
     // diagnostics (NULL: off): CLOCK_PROBE_WORKGROUPS x 4 cells in which the large-tile kernels note, per workgroup, the shader
     // clock counter and the 100 MHz counter at its start and at its end
     uint64_t*       clock_probe;

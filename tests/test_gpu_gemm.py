@@ -253,6 +253,91 @@ def test_fp8_four_wavefront_form_vs_oracle(calc, orc, policy, M, N, K, op, dtA, 
         assert np.array_equal(fused.cpu().numpy().view(codes.dtype), codes)
 
 
+@pytest.mark.parametrize("op,dtA,bA,mA,dtB,bB,mB,fused", [
+    (abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # exponent-15 codes are inf / NaN for Gaudi, 256 .. 448 for the hardware
+    (abi.OP_ABT, abi.FP8_143, 11, 1, abi.FP8_152, 15, 2, False),  # 0x7F is a number for Gaudi; exponent-31 codes likewise
+    (abi.OP_AB, abi.FP8_152, 15, 0, abi.FP8_143, 3, 0, False),    # fp8_152 in full mode is the hardware's format: its inf / NaN only end the fast conversions
+])
+def test_fp8_four_wavefront_form_recomputes_tiles_with_special_codes(calc, orc, op, dtA, bA, mA, dtB, bB, mB, fused):
+    """The four-wavefront form looks at every operand byte of its own tile in the fragment registers; a workgroup that meets a
+    code the matrix cores read differently computes its tile once more from exactly decoded operands, inside the same
+    launch.  One such code at a time, at positions that fall to different tiles, wavefronts, fragments and stages (first and
+    last included), in A or in B: the affected rows / columns and a slab elsewhere against the oracle, inf / NaN placement
+    included; clean operands afterwards give finite results again."""
+    import torch
+    M, N, K = 3072, 4096, 3072
+    rng = np.random.default_rng(9)
+    a0 = (rng.integers(0, 0x58, M * K).astype(np.uint8) | (rng.integers(0, 2, M * K).astype(np.uint8) << 7)).reshape(M, K)
+    b_rows, b_cols = (N, K) if op == abi.OP_ABT else (K, N)
+    b0 = (rng.integers(0, 0x58, K * N).astype(np.uint8) | (rng.integers(0, 2, K * N).astype(np.uint8) << 7)).reshape(b_rows, b_cols)
+    code_a = {0: [0x78, 0x7D, 0xF8], 1: [0x7F, 0xFF], 2: [0x7F]}[mA] if dtA == abi.FP8_143 else {0: [0x7C, 0xFD], 1: [0x7C, 0xFE], 2: [0x7D]}[mA]
+    code_b = {0: [0xF8, 0x7B], 1: [0x7F], 2: [0x7F]}[mB] if dtB == abi.FP8_143 else {0: [0x7C], 1: [0x7C, 0xFE], 2: [0x7D, 0xFC]}[mB]
+    # (which, f index, k index): rows of A / columns of B in different tiles and quarters of a tile, k in different stages
+    places = [("a", 0, 0), ("a", M - 1, K - 1), ("a", 300, 64 * 3 + 17), ("a", 5 * 256 + 129, 64 * 20 + 63), ("a", 7 * 256 + 70, K - 65),
+              ("b", 0, 0), ("b", N - 1, K - 1), ("b", 700, 64 * 2 + 5), ("b", 9 * 256 + 200, 64 * 31), ("b", 13 * 256 + 64, K - 64)]
+    asz, bsz = _shapes(op, M, N, K)
+    ta, tb = torch.from_numpy(a0.ravel().copy()).cuda(), torch.from_numpy(b0.ravel().copy()).cuda()
+    out = torch.zeros(M * N, dtype=torch.int16 if fused else torch.float32, device="cuda")
+    X, Wt, Y = MmeSimTensor(asz, 2, dtA, ta, bA, mA), MmeSimTensor(bsz, 2, dtB, tb, bB, mB), MmeSimTensor([N, M], 2, abi.BF16 if fused else abi.FP32, out)
+    epi = Epilogue(scale_exp=-4) if fused else None
+
+    def result():
+        calc.doBatchGemm(Y, X, Wt, op, epilogue=epi)
+        form = calc.lastContractionForm()
+        assert form["large_tile"] and form["wavefronts"] == 4 and form["split_k"] == 1, form
+        calc.synchronize()
+        r = out.cpu().numpy()
+        return (bf16_bits_to_f32(r.view(np.uint16)) if fused else r).reshape(M, N)
+
+    def expected(acc):
+        if not fused:
+            return acc
+        codes = np.zeros(acc.size, np.uint16)
+        assert orc.orc_cast_from_fp32(codes.ctypes.data, abi.BF16, 0, 0, acc.ctypes.data, acc.size, -4, None, 0, 0, 0, 0, 0, 0) == 0
+        return bf16_bits_to_f32(codes)
+
+    def reference_rows(a, b, rows):
+        want = np.zeros(rows.size * N, np.float32)
+        slab = np.ascontiguousarray(a[rows].ravel())
+        assert orc.orc_batch_gemm(A(desc(want, [N, rows.size], abi.FP32)), A(desc(slab, [K, rows.size], dtA, bA, mA)), A(desc(b.ravel(), bsz, dtB, bB, mB)), op) == 0
+        return expected(want).reshape(rows.size, N)
+
+    tol = 2e-3 if fused else 1e-4
+    n_checked = n_nonfinite = 0
+    for i, (which, fi, ki) in enumerate(places):
+        codes = code_a if which == "a" else code_b
+        code = codes[i % len(codes)]
+        a, b = a0.copy(), b0.copy()
+        if which == "a":
+            a[fi, ki] = code
+        elif op == abi.OP_ABT:
+            b[fi, ki] = code
+        else:
+            b[ki, fi] = code
+        ta.copy_(torch.from_numpy(a.ravel()))
+        tb.copy_(torch.from_numpy(b.ravel()))
+        got = result()
+        # the affected row (A), or rows of three different tile rows that all cross the affected column (B), plus six others
+        rows = np.unique(np.concatenate([[fi] if which == "a" else [1, M // 2 + 3, M - 2], rng.choice(M, 6, replace=False)]))
+        want = reference_rows(a, b, rows)
+        g = got[rows]
+        assert np.array_equal(np.isnan(g), np.isnan(want)), (which, fi, ki, hex(code))
+        inf = np.isinf(want)
+        assert np.array_equal(g[inf], want[inf]), (which, fi, ki, hex(code))
+        fin = np.isfinite(want)
+        assert rel_frobenius(g[fin], want[fin]) <= tol, (which, fi, ki, hex(code))
+        n_nonfinite += int((~fin).any())
+        n_checked += 1
+    assert n_checked == len(places)
+    if mA == 0 or mB == 0:
+        assert n_nonfinite >= 3
+    ta.copy_(torch.from_numpy(a0.ravel()))
+    tb.copy_(torch.from_numpy(b0.ravel()))
+    got = result()
+    rows = np.arange(16)
+    assert np.isfinite(got).all() and rel_frobenius(got[rows].ravel(), reference_rows(a0, b0, rows).ravel()) <= tol
+
+
 def test_fp8_short_reductions_keep_eight_wavefronts(calc):
     """Below 48 stages per workgroup, or with more tiles than one round, the form with eight wavefronts stays."""
     import torch
