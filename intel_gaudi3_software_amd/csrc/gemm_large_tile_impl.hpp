@@ -655,8 +655,9 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         {
             // the block-scale operands are exponents (2^(byte - 127), byte 0 of the register): the first carries the
             // epilogue's power-of-two factor when the host folded it in, the second is 2^0
-            // (only in the plain instance, see gemm_large_tile_takes_mfma_scale: with the scale operands the register allocator
-            // spills accumulators in the instances that walk over tiles or check their operands)
+            // (only in the plain instances, see gemm_large_tile_takes_mfma_scale: with the scale operands the register allocator
+            // spills in the instances that walk over tiles or check their operands -- also in the four-wavefront checking
+            // instance, 16 registers, which cost it more than the multiplication in the epilogue that the scale operand saves)
             if constexpr (!MSCALE) acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, 0, 0, 0);
             else
                 acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[j], f.a[i], acc[i][j], (FMT >> 1) & 1, FMT & 1, 0, mfma_scale_a, 0, 127);

@@ -554,6 +554,15 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     // promise, or the checks below), the accumulators stay below 2^(log2 K + 26) in the hardware formats' units, and the only
     // factor is the one power of two known here: the fast converters then skip their look-out for such values.
     const bool in_kernel_check = need_scan && gemm_large_tile_checks_operands(g);
+    // the four-wavefront form settles special codes inside its launch (panel words, see GemmProblem::chk_state); it needs those
+    // words, which the allocation-free entry point does not have: that one takes the eight-wavefront form
+    const size_t panel_words = (size_t) g.batch[0] * g.batch[1] * g.batch[2] * 2u * (size_t) (g.M / 256 + g.N / 256);
+    const bool   in_launch_check = in_kernel_check && g.waves == 4 && !h->noalloc && panel_words <= CHK_STATE_REGION_WORDS;
+    if (in_kernel_check && g.waves == 4 && !in_launch_check)
+    {
+        g.waves = 8;
+        h->last_form[3] = 8;
+    }
     {
         bool finite = h->fp8_specials_policy == MME_HIP_FP8_SPECIALS_ASSUME_NONE || in_kernel_check ||
                       (plan.nonfinite_kind[0] < 0 && plan.nonfinite_kind[1] < 0 && need_scan);
@@ -597,27 +606,16 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         g.chk_mask_a = mask[0], g.chk_add_a = add[0], g.chk_mask_b = mask[1], g.chk_add_b = add[1];
         g.chk_inf_nan_a = ta->inf_nan_mode, g.chk_inf_nan_b = tb->inf_nan_mode;
     };
-    if (in_kernel_check && g.waves == 4)
+    if (in_launch_check)
     {
-        // the four-wavefront form settles the matter inside its launch (panel words, see GemmProblem::chk_state); it needs
-        // those words, which the allocation-free entry point does not have: that one takes the eight-wavefront form
-        const size_t words = (size_t) g.batch[0] * g.batch[1] * g.batch[2] * 2u * (size_t) (g.M / 256 + g.N / 256);
-        if (h->noalloc || words > CHK_STATE_REGION_WORDS)
-        {
-            g.waves = 8;
-            h->last_form[3] = 8;
-        }
-        else
-        {
-            if (!h->chk_state.p) HIP_TRY(h, h->chk_state.reserve((size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS * sizeof(uint32_t)));
-            const unsigned slot = h->chk_state_launches++ % CHK_STATE_RING;
-            if (slot == 0) HIP_TRY(h, launch_fill_u32((uint32_t*) h->chk_state.p, 0u, (size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS, h->stream));
-            g.chk = 2;
-            g.chk_state = (uint32_t*) h->chk_state.p + (size_t) slot * CHK_STATE_REGION_WORDS;
-            set_check_constants();
-            HIP_TRY(h, launch_gemm(g, h->stream));
-            return MME_HIP_OK;
-        }
+        if (!h->chk_state.p) HIP_TRY(h, h->chk_state.reserve((size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS * sizeof(uint32_t)));
+        const unsigned slot = h->chk_state_launches++ % CHK_STATE_RING;
+        if (slot == 0) HIP_TRY(h, launch_fill_u32((uint32_t*) h->chk_state.p, 0u, (size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS, h->stream));
+        g.chk = 2;
+        g.chk_state = (uint32_t*) h->chk_state.p + (size_t) slot * CHK_STATE_REGION_WORDS;
+        set_check_constants();
+        HIP_TRY(h, launch_gemm(g, h->stream));
+        return MME_HIP_OK;
     }
     // the flag holds the epoch of the latest call that met such a code; the native kernel either finds them itself while it
     // multiplies (the large-tile kernels that can) or is skipped when a scan launch in front of it found one; decode + bf16
