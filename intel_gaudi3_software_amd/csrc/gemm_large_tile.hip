@@ -227,11 +227,18 @@ int gemm_fast_pick_tile_m(const GemmProblem& p, int num_cus)
 // tiles need several rounds (8192 x 8192 x 4096).  So: one round of tiles and at least 48 stages per workgroup.
 int gemm_fast_pick_waves(const GemmProblem& p, int num_cus)
 {
-    if (!gemm_large_tile_checks_operands(p) || gemm_large_tile_persistent_applicable(p)) return 8;
     // (one round: with half as many tiles or fewer the 128-row tiles take over, with more than one round's worth nothing is
     // split, so this form never meets split-k)
-    const long long groups = (long long) (p.M / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2];
-    return p.split_k <= 1 && groups <= num_cus && p.K / FBK >= 48 ? 4 : 8;
+    return gemm_large_tile_one_round(p, num_cus) && p.K / FBK >= 48 ? 4 : 8;
+}
+
+// An fp8 GEMM of whole 256-row tiles, one workgroup per tile (not the persistent walk, no split-k), whose workgroups are all
+// resident at once on a device that does nothing else: the checking instances may then settle special codes among themselves
+// (GemmProblem::chk == 2).
+bool gemm_large_tile_one_round(const GemmProblem& p, int num_cus)
+{
+    if (!gemm_large_tile_checks_operands(p) || gemm_large_tile_persistent_applicable(p) || p.split_k > 1) return false;
+    return (long long) (p.M / FBM) * (p.N / FBN) * p.batch[0] * p.batch[1] * p.batch[2] <= num_cus;
 }
 
 int gemm_fast_pick_split_k(const GemmProblem& p, int num_cus)

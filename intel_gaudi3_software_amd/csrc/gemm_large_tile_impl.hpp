@@ -218,12 +218,13 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     constexpr bool RAGGED_M = AMODE == 1 || AMODE == 3 || RG; // the last row tile may be partial
     // (RG: the last column tile may be partial too; N is a multiple of 16, so a lane's 16 columns are all in or all out)
     constexpr bool A_KC = AMODE < 2;
-    // CHK with four wavefronts (one round of tiles, every workgroup resident): the workgroups take turns at looking like the
-    // eight-wavefront forms do, but note per operand panel what they found and how many of a panel's lookers are done; after its
-    // epilogue a workgroup waits for the lookers of its own two panels (long done by then) and, if one of them met such a code,
-    // computes its tile once more, exactly, inside the same launch (below, after the loop).  No flag for the host, nothing
-    // enqueued behind the kernel.
-    constexpr bool SELFCHK = CHK && NW == 4;
+    // CHK, one workgroup per tile: when the host says so (chk == 2: one round of tiles, every workgroup resident) the workgroups
+    // note per operand panel what their looks found and how many of a panel's lookers are done; after its epilogue a workgroup
+    // waits for the lookers of its own two panels (long done by then) and, if one of them met such a code, computes its tile
+    // once more, exactly, inside the same launch (below, after the loop).  No flag for the host then, nothing enqueued behind
+    // the kernel.
+    constexpr bool SELFCHK = CHK && !PERSIST;
+    const bool     in_launch = SELFCHK && g.chk == 2;
     extern __shared__ __attribute__((aligned(1024))) char lds[];
     warm_kernargs(g);
     if (!CHK && g.skip_flag && ((*g.skip_flag == g.skip_epoch) == (g.skip_if != 0))) return;
@@ -867,10 +868,13 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
 #undef RB
 #undef LA
 #undef LB
-    if constexpr (CHK && !SELFCHK)
+    if constexpr (CHK)
     {
-        if (chk_bad & 0x80808080u) *const_cast<uint32_t*>((const uint32_t*) g.skip_flag) = g.skip_epoch;
-        chk_bad = 0;
+        if (!in_launch)
+        {
+            if ((chk_bad | chk_bad_b) & 0x80808080u) *const_cast<uint32_t*>((const uint32_t*) g.skip_flag) = g.skip_epoch;
+            chk_bad = 0;
+        }
     }
     // SELFCHK: what this workgroup's looks found goes into the launch's panel words (GemmProblem::chk_state, zero before the
     // launch; per batch element: a flag per row panel of A, a flag per column panel of B, then a count of finished lookers
@@ -880,7 +884,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     uint32_t* panel_flag_b = nullptr;
     uint32_t* panel_done_a = nullptr;
     uint32_t* panel_done_b = nullptr;
-    if constexpr (SELFCHK)
+    if (in_launch)
     {
         uint32_t* st = g.chk_state + (size_t) blockIdx.y * 2u * (unsigned) (tiles_m + tiles_n);
         panel_flag_a = st + cur_tm;
@@ -1291,7 +1295,7 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
     }
     else if (!PERSIST)
         store_generic();
-    if constexpr (SELFCHK)
+    if (in_launch)
     {
         // every looker of this tile's row panel of A (one workgroup per tile column) and of its column panel of B has finished
         // its loop before it started the epilogue that this workgroup has just finished as well, so the wait is a formality

@@ -554,15 +554,10 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     // promise, or the checks below), the accumulators stay below 2^(log2 K + 26) in the hardware formats' units, and the only
     // factor is the one power of two known here: the fast converters then skip their look-out for such values.
     const bool in_kernel_check = need_scan && gemm_large_tile_checks_operands(g);
-    // the four-wavefront form settles special codes inside its launch (panel words, see GemmProblem::chk_state); it needs those
-    // words, which the allocation-free entry point does not have: that one takes the eight-wavefront form
+    // a launch whose workgroups are all resident at once settles special codes inside the launch (panel words, see
+    // GemmProblem::chk_state); it needs those words, which the allocation-free entry point does not have
     const size_t panel_words = (size_t) g.batch[0] * g.batch[1] * g.batch[2] * 2u * (size_t) (g.M / 256 + g.N / 256);
-    const bool   in_launch_check = in_kernel_check && g.waves == 4 && !h->noalloc && panel_words <= CHK_STATE_REGION_WORDS;
-    if (in_kernel_check && g.waves == 4 && !in_launch_check)
-    {
-        g.waves = 8;
-        h->last_form[3] = 8;
-    }
+    const bool   in_launch_check = in_kernel_check && gemm_large_tile_one_round(g, h->num_cus) && !h->noalloc && panel_words <= CHK_STATE_REGION_WORDS;
     {
         bool finite = h->fp8_specials_policy == MME_HIP_FP8_SPECIALS_ASSUME_NONE || in_kernel_check ||
                       (plan.nonfinite_kind[0] < 0 && plan.nonfinite_kind[1] < 0 && need_scan);

@@ -169,6 +169,7 @@ hipError_t launch_gemm(const GemmProblem& p, hipStream_t s);
 bool       gemm_large_tile_applicable(const GemmProblem& p);
 int        gemm_fast_pick_split_k(const GemmProblem& p, int num_cus); // 0: the large-tile kernel does not take this problem
 int        gemm_fast_pick_waves(const GemmProblem& p, int num_cus);   // (after tile_m and split_k have been chosen)
+bool       gemm_large_tile_one_round(const GemmProblem& p, int num_cus); // (likewise)
 hipError_t launch_gemm_large_tile(const GemmProblem& p, hipStream_t s);
 // the kernel this problem takes can check its fp8 operands for special codes itself (GemmProblem::chk)
 bool       gemm_large_tile_checks_operands(const GemmProblem& p);

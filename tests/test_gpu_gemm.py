@@ -253,19 +253,22 @@ def test_fp8_four_wavefront_form_vs_oracle(calc, orc, policy, M, N, K, op, dtA, 
         assert np.array_equal(fused.cpu().numpy().view(codes.dtype), codes)
 
 
-@pytest.mark.parametrize("op,dtA,bA,mA,dtB,bB,mB,fused", [
-    (abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # exponent-15 codes are inf / NaN for Gaudi, 256 .. 448 for the hardware
-    (abi.OP_ABT, abi.FP8_143, 11, 1, abi.FP8_152, 15, 2, False),  # 0x7F is a number for Gaudi; exponent-31 codes likewise
-    (abi.OP_AB, abi.FP8_152, 15, 0, abi.FP8_143, 3, 0, False),    # fp8_152 in full mode is the hardware's format: its inf / NaN only end the fast conversions
+@pytest.mark.parametrize("K,op,dtA,bA,mA,dtB,bB,mB,fused", [
+    (3072, abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # exponent-15 codes are inf / NaN for Gaudi, 256 .. 448 for the hardware
+    (3072, abi.OP_ABT, abi.FP8_143, 11, 1, abi.FP8_152, 15, 2, False),  # 0x7F is a number for Gaudi; exponent-31 codes likewise
+    (3072, abi.OP_AB, abi.FP8_152, 15, 0, abi.FP8_143, 3, 0, False),    # fp8_152 in full mode is the hardware's format: its inf / NaN only end the fast conversions
+    (1024, abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # a short reduction: the form with eight wavefronts, still one round of tiles
+    (1024, abi.OP_ABT, abi.FP8_143, 3, 0, abi.FP8_152, 15, 1, False),
 ])
-def test_fp8_four_wavefront_form_recomputes_tiles_with_special_codes(calc, orc, op, dtA, bA, mA, dtB, bB, mB, fused):
-    """The four-wavefront form looks at every operand byte of its own tile in the fragment registers; a workgroup that meets a
-    code the matrix cores read differently computes its tile once more from exactly decoded operands, inside the same
-    launch.  One such code at a time, at positions that fall to different tiles, wavefronts, fragments and stages (first and
-    last included), in A or in B: the affected rows / columns and a slab elsewhere against the oracle, inf / NaN placement
-    included; clean operands afterwards give finite results again."""
+def test_fp8_one_round_launches_recompute_tiles_with_special_codes(calc, orc, K, op, dtA, bA, mA, dtB, bB, mB, fused):
+    """When the tiles of an fp8 GEMM make one round (3072 x 4096 outputs = 192 workgroups), the workgroups share per operand
+    panel what their looks at the operand bytes found, and a workgroup whose panels hold a code that the matrix cores read
+    differently computes its tile once more from exactly decoded operands, inside the same launch.  One such code at a time,
+    at positions that fall to different tiles, wavefronts and stages (first and last included), in A or in B: the affected
+    rows / columns and a slab elsewhere against the oracle, inf / NaN placement included; clean operands afterwards give finite
+    results again.  Both forms of the kernel (four wavefronts for the long reduction, eight for the short one)."""
     import torch
-    M, N, K = 3072, 4096, 3072
+    M, N = 3072, 4096
     rng = np.random.default_rng(9)
     a0 = (rng.integers(0, 0x58, M * K).astype(np.uint8) | (rng.integers(0, 2, M * K).astype(np.uint8) << 7)).reshape(M, K)
     b_rows, b_cols = (N, K) if op == abi.OP_ABT else (K, N)
@@ -273,8 +276,8 @@ def test_fp8_four_wavefront_form_recomputes_tiles_with_special_codes(calc, orc, 
     code_a = {0: [0x78, 0x7D, 0xF8], 1: [0x7F, 0xFF], 2: [0x7F]}[mA] if dtA == abi.FP8_143 else {0: [0x7C, 0xFD], 1: [0x7C, 0xFE], 2: [0x7D]}[mA]
     code_b = {0: [0xF8, 0x7B], 1: [0x7F], 2: [0x7F]}[mB] if dtB == abi.FP8_143 else {0: [0x7C], 1: [0x7C, 0xFE], 2: [0x7D, 0xFC]}[mB]
     # (which, f index, k index): rows of A / columns of B in different tiles and quarters of a tile, k in different stages
-    places = [("a", 0, 0), ("a", M - 1, K - 1), ("a", 300, 64 * 3 + 17), ("a", 5 * 256 + 129, 64 * 20 + 63), ("a", 7 * 256 + 70, K - 65),
-              ("b", 0, 0), ("b", N - 1, K - 1), ("b", 700, 64 * 2 + 5), ("b", 9 * 256 + 200, 64 * 31), ("b", 13 * 256 + 64, K - 64)]
+    places = [("a", 0, 0), ("a", M - 1, K - 1), ("a", 300, 64 * 3 + 17), ("a", 5 * 256 + 129, 64 * (K // 150) + 63), ("a", 7 * 256 + 70, K - 65),
+              ("b", 0, 0), ("b", N - 1, K - 1), ("b", 700, 64 * 2 + 5), ("b", 9 * 256 + 200, 64 * (K // 100)), ("b", 13 * 256 + 64, K - 64)]
     asz, bsz = _shapes(op, M, N, K)
     ta, tb = torch.from_numpy(a0.ravel().copy()).cuda(), torch.from_numpy(b0.ravel().copy()).cuda()
     out = torch.zeros(M * N, dtype=torch.int16 if fused else torch.float32, device="cuda")
@@ -284,7 +287,7 @@ def test_fp8_four_wavefront_form_recomputes_tiles_with_special_codes(calc, orc, 
     def result():
         calc.doBatchGemm(Y, X, Wt, op, epilogue=epi)
         form = calc.lastContractionForm()
-        assert form["large_tile"] and form["wavefronts"] == 4 and form["split_k"] == 1, form
+        assert form["large_tile"] and form["wavefronts"] == (4 if K >= 3072 else 8) and form["split_k"] == 1 and form["tile_rows"] == 256, form
         calc.synchronize()
         r = out.cpu().numpy()
         return (bf16_bits_to_f32(r.view(np.uint16)) if fused else r).reshape(M, N)
