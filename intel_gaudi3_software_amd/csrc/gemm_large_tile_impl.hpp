@@ -876,34 +876,26 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             chk_bad = 0;
         }
     }
-    // SELFCHK: what this workgroup's looks found goes into the launch's panel words (GemmProblem::chk_state, zero before the
-    // launch; per batch element: a flag per row panel of A, a flag per column panel of B, then a count of finished lookers
-    // for each), the flags before the counts, all with device scope.
+    // In-launch settling: what this workgroup's looks found goes into the launch's panel words (GemmProblem::chk_state, zero
+    // before the launch; per batch element one word per row panel of A, then one per column panel of B): one device-scope
+    // addition per panel that counts this workgroup as a finished looker in the low half of the word and a find in the high
+    // half.  Count and flag travel together, so a reader needs one look per panel and no ordering between words.  (Relaxed
+    // accesses: the words are the only data that pass between workgroups, there is nothing for a release to write back or
+    // an acquire to invalidate -- with release / acquire every workgroup flushed and invalidated its L2, 2 us per launch.)
     bool      tile_exact = false;
-    uint32_t* panel_flag_a = nullptr;
-    uint32_t* panel_flag_b = nullptr;
-    uint32_t* panel_done_a = nullptr;
-    uint32_t* panel_done_b = nullptr;
+    uint32_t* panel_a = nullptr;
+    uint32_t* panel_b = nullptr;
     if (in_launch)
     {
-        uint32_t* st = g.chk_state + (size_t) blockIdx.y * 2u * (unsigned) (tiles_m + tiles_n);
-        panel_flag_a = st + cur_tm;
-        panel_flag_b = st + tiles_m + cur_tn;
-        panel_done_a = st + tiles_m + tiles_n + cur_tm;
-        panel_done_b = st + 2 * tiles_m + tiles_n + cur_tn;
+        uint32_t* st = g.chk_state + (size_t) blockIdx.y * (unsigned) (tiles_m + tiles_n);
+        panel_a = st + cur_tm;
+        panel_b = st + tiles_m + cur_tn;
         const bool bad_a = __syncthreads_or((chk_bad & 0x80808080u) != 0u) != 0, bad_b = __syncthreads_or((chk_bad_b & 0x80808080u) != 0u) != 0;
         chk_bad = 0;
         if (threadIdx.x == 0)
         {
-            // (relaxed device-scope accesses, ordered by hand: the flags are the only data that pass between workgroups, so there
-            // is nothing for a release to write back and nothing for an acquire to invalidate -- with release / acquire every
-            // workgroup flushed and invalidated its L2, 2 us per launch; the wait lets the flag stores be acknowledged before the
-            // counts go out)
-            if (bad_a) __hip_atomic_store(panel_flag_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (bad_b) __hip_atomic_store(panel_flag_b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (bad_a || bad_b) __builtin_amdgcn_s_waitcnt(vm_wait(0));
-            __hip_atomic_fetch_add(panel_done_a, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_fetch_add(panel_done_b, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(panel_a, 1u + (bad_a ? 0x10000u : 0u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(panel_b, 1u + (bad_b ? 0x10000u : 0u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     // The tile once more, from operands decoded to bf16 with Gaudi's meaning of the codes (every fp8 value is a bf16 value;
@@ -1303,15 +1295,16 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
         bool again = false;
         if (threadIdx.x == 0)
         {
-            bool all_in = false;
+            bool     all_in = false;
+            uint32_t wa = 0, wb = 0;
             for (int polls = 0; polls < (1 << 14) && !all_in; polls++)
             {
-                all_in = __hip_atomic_load(panel_done_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t) tiles_n &&
-                         __hip_atomic_load(panel_done_b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t) tiles_m;
+                wa = __hip_atomic_load(panel_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                wb = __hip_atomic_load(panel_b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                all_in = (wa & 0xFFFFu) >= (uint32_t) tiles_n && (wb & 0xFFFFu) >= (uint32_t) tiles_m;
                 if (!all_in) __builtin_amdgcn_s_sleep(16);
             }
-            again = !all_in || __hip_atomic_load(panel_flag_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u ||
-                    __hip_atomic_load(panel_flag_b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+            again = !all_in || ((wa | wb) >> 16) != 0u;
         }
         if (__builtin_expect(__syncthreads_or(again) != 0, 0))
         {

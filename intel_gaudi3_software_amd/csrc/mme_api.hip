@@ -89,7 +89,7 @@ struct mme_hip_calc
     uint32_t              specials_epoch = 0; // epoch number of the latest call that scanned
     int                   fp8_specials_policy = 0;
     int                   last_form[4] = {0, 256, 1, 8}; // mme_hip_last_contraction_form
-    // panel words of the four-wavefront checking GEMM (GemmProblem::chk_state): a ring of regions, one per launch, all cleared by
+    // panel words of the fp8 GEMMs that settle special codes inside their launch (GemmProblem::chk_state): a ring of regions, one per launch, all cleared by
     // one fill launch every CHK_STATE_RING launches
     DeviceBuffer          chk_state;
     unsigned              chk_state_launches = 0;
@@ -131,8 +131,8 @@ int hip_fail(mme_hip_handle h, hipError_t e, const char* what)
 
 // Work space of `bytes` for the current call: the handle's grow-only buffer `buf`, or, in a call that may not allocate, the
 // next piece of the device's static scratch array.
-// panel words of the four-wavefront checking GEMM: words per launch (2 x (row panels + column panels) per batch element, at
-// most 256 tiles in all) and launches per clearing
+// panel words of the fp8 GEMMs that settle special codes inside their launch: words per launch (row panels + column panels per
+// batch element, at most 256 tiles in all) and launches per clearing
 constexpr size_t   CHK_STATE_REGION_WORDS = 2048;
 constexpr unsigned CHK_STATE_RING = 64;
 
@@ -556,7 +556,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     const bool in_kernel_check = need_scan && gemm_large_tile_checks_operands(g);
     // a launch whose workgroups are all resident at once settles special codes inside the launch (panel words, see
     // GemmProblem::chk_state); it needs those words, which the allocation-free entry point does not have
-    const size_t panel_words = (size_t) g.batch[0] * g.batch[1] * g.batch[2] * 2u * (size_t) (g.M / 256 + g.N / 256);
+    const size_t panel_words = (size_t) g.batch[0] * g.batch[1] * g.batch[2] * (size_t) (g.M / 256 + g.N / 256);
     const bool   in_launch_check = in_kernel_check && gemm_large_tile_one_round(g, h->num_cus) && !h->noalloc && panel_words <= CHK_STATE_REGION_WORDS;
     {
         bool finite = h->fp8_specials_policy == MME_HIP_FP8_SPECIALS_ASSUME_NONE || in_kernel_check ||

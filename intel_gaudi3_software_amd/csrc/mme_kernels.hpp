@@ -141,7 +141,7 @@ struct GemmProblem
     uint32_t        chk_mask_a, chk_add_a, chk_mask_b, chk_add_b; // the byte constants replicated over a 32-bit word
     // The four-wavefront form (chk == 2; one round of tiles, every workgroup resident) settles the matter inside the launch: the
     // looks are shared out the same way, but what they find is noted per operand panel in chk_state (zero before the launch,
-    // 2 x (row panels + column panels) words per batch element: flags, then counts of finished lookers), and a workgroup
+    // row panels + column panels words per batch element: finished lookers in the low half, finds in the high half), and a workgroup
     // whose panels hold such a code computes its tile once more, exactly, from operands decoded with Gaudi's meaning of the
     // codes (inf / NaN modes below; the hardware formats' exponent bias, so that the epilogue's factor stays the same).
     int             chk_inf_nan_a, chk_inf_nan_b;
