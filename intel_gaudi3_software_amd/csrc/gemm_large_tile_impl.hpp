@@ -1299,8 +1299,10 @@ __device__ __forceinline__ void gemm_fast_body_impl(KARG GemmProblem& g)
             uint32_t wa = 0, wb = 0;
             for (int polls = 0; polls < (1 << 14) && !all_in; polls++)
             {
-                wa = __hip_atomic_load(panel_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                wb = __hip_atomic_load(panel_b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // (read with an addition of zero: a read-modify-write is carried out where all XCDs agree, whatever a plain load
+                // with device scope may find in this XCD's L2)
+                wa = __hip_atomic_fetch_add(panel_a, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                wb = __hip_atomic_fetch_add(panel_b, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 all_in = (wa & 0xFFFFu) >= (uint32_t) tiles_n && (wb & 0xFFFFu) >= (uint32_t) tiles_m;
                 if (!all_in) __builtin_amdgcn_s_sleep(16);
             }
