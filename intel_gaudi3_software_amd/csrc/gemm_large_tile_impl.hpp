@@ -186,7 +186,9 @@ __device__ __attribute__((aligned(16))) uint32_t gf_zero_page[GF_ZERO_PAGE_BYTES
 // meets one.  Every 64-byte stage of an operand row is looked at by exactly one of the workgroups that read it (stage t of
 // the A rows by the tile column t mod tiles_n, of the B columns by the tile row t mod tiles_m): when its turn comes, each
 // wavefront reads an eighth of that part of the stage once more from LDS and tests the bytes, a few vector instructions in
-// the shadow of the matrix instructions, so a clean operand costs no extra pass over memory and no extra launch.
+// the shadow of the matrix instructions, so a clean operand costs no extra pass over memory and no extra launch.  With one
+// workgroup per tile and one round of tiles (GemmProblem::chk == 2) the hit is not handed to the host's fall-back but
+// settled inside the launch: see SELFCHK in the body.
 // NST: stages of the ring (4 to 6, default 4; every instantiation uses the default: six stages of the 128-row tile's 24 KiB
 // measured 2-3 % slower than four on the 3 x 3 convolutions of 32 x 28 x 28 x 256, whose steps then divide by six to find a slot).
 // The reduction has to be at least NST stages long.
