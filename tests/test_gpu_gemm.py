@@ -341,6 +341,43 @@ def test_fp8_one_round_launches_recompute_tiles_with_special_codes(calc, orc, K,
     assert np.isfinite(got).all() and rel_frobenius(got[rows].ravel(), reference_rows(a0, b0, rows).ravel()) <= tol
 
 
+@pytest.mark.parametrize("K", [3072, 1024])
+def test_fp8_one_round_launch_with_batches_settles_special_codes_per_batch_element(calc, orc, K):
+    """Two batch elements of 1536 x 4096 outputs (2 x 96 tiles: one round), A per batch element, B shared: the panel words in
+    which the workgroups share their finds are kept per batch element.  A special code in batch element 1 of A, and one in
+    the shared B: the first changes rows of batch element 1 only, the second columns of both; everything against the oracle."""
+    import torch
+    M, N = 1536, 4096
+    rng = np.random.default_rng(31)
+    a = (rng.integers(0, 0x58, 2 * M * K).astype(np.uint8) | (rng.integers(0, 2, 2 * M * K).astype(np.uint8) << 7)).reshape(2, M, K)
+    b = (rng.integers(0, 0x58, K * N).astype(np.uint8) | (rng.integers(0, 2, K * N).astype(np.uint8) << 7)).reshape(K, N)
+    a[1, 700, K - 3] = 0x78      # +inf for Gaudi's fp8_143 in full mode
+    b[64 * 5 + 9, 2049] = 0x7D   # NaN
+    ta, tb = torch.from_numpy(a.ravel().copy()).cuda(), torch.from_numpy(b.ravel().copy()).cuda()
+    out = torch.zeros(2 * M * N, dtype=torch.float32, device="cuda")
+    calc.doBatchGemm(MmeSimTensor([N, M, 2, 1, 1], 5, abi.FP32, out), MmeSimTensor([K, M, 2, 1, 1], 5, abi.FP8_143, ta, 7),
+                     MmeSimTensor([N, K, 1, 1, 1], 5, abi.FP8_143, tb, 7), abi.OP_AB)
+    form = calc.lastContractionForm()
+    assert form["large_tile"] and form["tile_rows"] == 256 and form["split_k"] == 1 and form["wavefronts"] == (4 if K >= 3072 else 8), form
+    calc.synchronize()
+    got = out.cpu().numpy().reshape(2, M, N)
+    rows = np.array([0, 5, 255, 256, 699, 700, 701, 1000, M - 1])
+    for bz in range(2):
+        want = np.zeros(rows.size * N, np.float32)
+        slab = np.ascontiguousarray(a[bz][rows].ravel())
+        assert orc.orc_batch_gemm(A(desc(want, [N, rows.size], abi.FP32)), A(desc(slab, [K, rows.size], abi.FP8_143, 7)), A(desc(b.ravel(), [N, K], abi.FP8_143, 7)), abi.OP_AB) == 0
+        want = want.reshape(rows.size, N)
+        g = got[bz][rows]
+        assert np.array_equal(np.isnan(g), np.isnan(want)) and np.array_equal(np.isinf(g), np.isinf(want)), bz
+        fin = np.isfinite(want)
+        assert np.array_equal(g[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+        assert rel_frobenius(g[fin], want[fin]) <= 1e-4
+        # column 2049 is NaN in every row of both batch elements, row 700 is not finite in batch element 1 only
+        assert np.isnan(got[bz][:, 2049]).all()
+        assert np.isfinite(np.delete(got[bz], 2049, axis=1)[np.arange(M) != 700]).all()
+    assert np.isfinite(np.delete(got[0][700], 2049)).all() and not np.isfinite(np.delete(got[1][700], 2049)).any()
+
+
 def test_fp8_short_reductions_keep_eight_wavefronts(calc):
     """Below 48 stages per workgroup, or with more tiles than one round, the form with eight wavefronts stays."""
     import torch
