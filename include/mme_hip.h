@@ -268,7 +268,8 @@ int mme_hip_set_operand_clip(mme_hip_handle h, int clip_fp, int clip_fp_inf_in);
  *   MME_HIP_FP8_SPECIALS_CHECK (default): operands in such modes are scanned on the device; if a scan finds such a
  *     code the contraction runs on an exact bf16 decode of the operands instead (the whole contraction, enqueued behind
  *     the native kernel and predicated on a device flag; or, for large one-round fp8 GEMMs, the affected output tiles
- *     only, inside the native kernel's own launch).  No host synchronisation.
+ *     only, inside the native kernel's own launch; calls enqueued while the stream records a graph always take the
+ *     predicated form, whose device flag survives replays on the safe side).  No host synchronisation.
  *   MME_HIP_FP8_SPECIALS_ASSUME_NONE: the caller guarantees that neither operand holds a code with all exponent bits set
  *     (e.g. the operands come out of a saturating quantiser, which never emits them); nothing is checked, and the
  *     output conversion does not look out for inf / NaN accumulators either.

@@ -557,7 +557,20 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     // a launch whose workgroups are all resident at once settles special codes inside the launch (panel words, see
     // GemmProblem::chk_state); it needs those words, which the allocation-free entry point does not have
     const size_t panel_words = (size_t) g.batch[0] * g.batch[1] * g.batch[2] * (size_t) (g.M / 256 + g.N / 256);
-    const bool   in_launch_check = in_kernel_check && gemm_large_tile_one_round(g, h->num_cus) && !h->noalloc && panel_words <= CHK_STATE_REGION_WORDS;
+    bool         in_launch_check = in_kernel_check && gemm_large_tile_one_round(g, h->num_cus) && !h->noalloc && panel_words <= CHK_STATE_REGION_WORDS;
+    if (in_launch_check)
+    {
+        // A launch recorded into a graph is replayed with the panel words as its last run left them, counts already at their
+        // final values: a workgroup would look at a panel before this run's lookers have reported.  Recorded calls take the
+        // epoch flag below, which a replay may find set by an earlier run (then the exact kernels run: slower, never wrong).
+        hipStreamCaptureStatus recording = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(h->stream, &recording) != hipSuccess)
+        {
+            (void) hipGetLastError();
+            recording = hipStreamCaptureStatusActive;
+        }
+        in_launch_check = recording == hipStreamCaptureStatusNone;
+    }
     {
         bool finite = h->fp8_specials_policy == MME_HIP_FP8_SPECIALS_ASSUME_NONE || in_kernel_check ||
                       (plan.nonfinite_kind[0] < 0 && plan.nonfinite_kind[1] < 0 && need_scan);
