@@ -209,7 +209,10 @@ int mme_hip_limit_num_of_threads(mme_hip_handle h, unsigned num_threads);
 /* The handle's hipStream_t as void*.  _dev calls are enqueued on it. */
 void* mme_hip_stream(mme_hip_handle h);
 
-/* Use a caller-owned hipStream_t (NULL = the handle's own stream). */
+/* Use a caller-owned hipStream_t (NULL = the handle's own stream).  A handle's work spaces (split-k partial sums, decoded
+ * operand copies, the flags and counters of the fp8 operand checks) are reused from call to call in stream order: the
+ * caller orders the new stream behind what the handle enqueued on the previous one (or waits for it) before the next call.
+ * Calls that may overlap in time belong on handles of their own. */
 int mme_hip_set_stream(mme_hip_handle h, void* hip_stream);
 
 /* hipStreamSynchronize on the handle's stream. */
