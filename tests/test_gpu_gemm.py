@@ -253,22 +253,25 @@ def test_fp8_four_wavefront_form_vs_oracle(calc, orc, policy, M, N, K, op, dtA, 
         assert np.array_equal(fused.cpu().numpy().view(codes.dtype), codes)
 
 
-@pytest.mark.parametrize("K,op,dtA,bA,mA,dtB,bB,mB,fused", [
-    (3072, abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # exponent-15 codes are inf / NaN for Gaudi, 256 .. 448 for the hardware
-    (3072, abi.OP_ABT, abi.FP8_143, 11, 1, abi.FP8_152, 15, 2, False),  # 0x7F is a number for Gaudi; exponent-31 codes likewise
-    (3072, abi.OP_AB, abi.FP8_152, 15, 0, abi.FP8_143, 3, 0, False),    # fp8_152 in full mode is the hardware's format: its inf / NaN only end the fast conversions
-    (1024, abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # a short reduction: the form with eight wavefronts, still one round of tiles
-    (1024, abi.OP_ABT, abi.FP8_143, 3, 0, abi.FP8_152, 15, 1, False),
+@pytest.mark.parametrize("M,K,op,dtA,bA,mA,dtB,bB,mB,fused", [
+    (3072, 3072, abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # exponent-15 codes are inf / NaN for Gaudi, 256 .. 448 for the hardware
+    (3072, 3072, abi.OP_ABT, abi.FP8_143, 11, 1, abi.FP8_152, 15, 2, False),  # 0x7F is a number for Gaudi; exponent-31 codes likewise
+    (3072, 3072, abi.OP_AB, abi.FP8_152, 15, 0, abi.FP8_143, 3, 0, False),    # fp8_152 in full mode is the hardware's format: its inf / NaN only end the fast conversions
+    (3072, 1024, abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),      # a short reduction: the form with eight wavefronts, still one round of tiles
+    (3072, 1024, abi.OP_ABT, abi.FP8_143, 3, 0, abi.FP8_152, 15, 1, False),
+    # 4096 x 4096 outputs: all 256 compute units busy, sixteen lookers per panel of either operand
+    (4096, 3072, abi.OP_AB, abi.FP8_143, 7, 0, abi.FP8_143, 7, 0, True),
+    (4096, 3072, abi.OP_ABT, abi.FP8_143, 11, 1, abi.FP8_152, 15, 2, False),
 ])
-def test_fp8_one_round_launches_recompute_tiles_with_special_codes(calc, orc, K, op, dtA, bA, mA, dtB, bB, mB, fused):
-    """When the tiles of an fp8 GEMM make one round (3072 x 4096 outputs = 192 workgroups), the workgroups share per operand
+def test_fp8_one_round_launches_recompute_tiles_with_special_codes(calc, orc, M, K, op, dtA, bA, mA, dtB, bB, mB, fused):
+    """When the tiles of an fp8 GEMM make one round (3072 x 4096 outputs = 192 workgroups, 4096 x 4096 = 256), the workgroups share per operand
     panel what their looks at the operand bytes found, and a workgroup whose panels hold a code that the matrix cores read
     differently computes its tile once more from exactly decoded operands, inside the same launch.  One such code at a time,
     at positions that fall to different tiles, wavefronts and stages (first and last included), in A or in B: the affected
     rows / columns and a slab elsewhere against the oracle, inf / NaN placement included; clean operands afterwards give finite
     results again.  Both forms of the kernel (four wavefronts for the long reduction, eight for the short one)."""
     import torch
-    M, N = 3072, 4096
+    N = 4096
     rng = np.random.default_rng(9)
     a0 = (rng.integers(0, 0x58, M * K).astype(np.uint8) | (rng.integers(0, 2, M * K).astype(np.uint8) << 7)).reshape(M, K)
     b_rows, b_cols = (N, K) if op == abi.OP_ABT else (K, N)
