@@ -31,11 +31,48 @@ PEAK_TFLOPS = {"fp8": 5000.0, "bf16": 2500.0, "fp32": 157.3}  # dense MFMA peaks
 PEAK_HBM_GBS = 8000.0
 METRIC = "TFLOP/s & % fp8/bf16 MFMA peak (GEMM, conv); cast GB/s vs HBM peak; 1 GPU"
 
-# HBM bytes per launch of each workload's kernels (fetched + written), from the FETCH_SIZE / WRITE_SIZE counter runs
-# summarised per workload under profiles/ (the headline GEMM: 101.2 MB fetched + 33.6 MB written for 67.1 MB algorithmic)
-GEMM_TRAFFIC_BYTES = 134.8e6
-TRAFFIC_BYTES = {"c1": 4.4e6, "c3": 54.9e6, "c4_dedx": 54.0e6, "c4_dedw": 71.9e6 + 35.5e6, "c5": 844.3e6, "cast_fp8_143": 1342.1e6,
-                 "cast_bf16": 1610.6e6, "dequant_fp8_143": 1342.4e6}
+# The rocprofv3 summary of each workload under profiles/ ends with a line "bench.py reads: kernel_us=... fetch_bytes=...
+# write_bytes=..." (traced average duration of the workload's kernels per call; bytes that crossed the L2 <-> memory
+# boundary per call, from the FETCH_SIZE / WRITE_SIZE counter runs).  roofline.traffic and roofline.profile come from that
+# line, so they change when the profile is taken again and are null when there is none.
+PROFILE_FILE = {"c2": "gemm_fp8_w4_kernel_fp8_gemm_4096x4096x4096.txt", "c1": "gemm_2byte_fast128_kernel_bf16_gemm_512x512x512.txt",
+                "c3": "conv_fwd_resident_kernel_bf16_conv_fwd_n64_56x56_c64_k64_3x3.txt",
+                "c4_dedx": "conv_2byte_fast128_kernel_bf16_conv_dedx_n32_28x28_c256_k256_3x3.txt",
+                "c4_dedw": "conv_dedw_2byte_fast128_kernel_bf16_conv_dedw_n32_28x28_c256_k256_3x3.txt",
+                "c5": "gemm_fp8_persistent_chk_kernel_fp8_batched_gemm_4x2048x4096x14336.txt",
+                "cast_fp8_143": "cast_from_fp32_kernel_fp32_to_fp8_143_2pow28.txt", "cast_bf16": "cast_from_fp32_kernel_fp32_to_bf16_2pow28.txt",
+                "dequant_fp8_143": "cast_to_fp32_kernel_fp8_143_to_fp32_2pow28.txt"}
+SETTLE_MS = 60
+ROTATE_BYTES = 320 << 20  # operand / output sets of the rotating variants cycle through at least this much memory (memory-side cache: 256 MiB)
+
+
+def profile_figures(name, work, peak):
+    """What the committed profile of workload `name` says: traced kernel time per call, the roofline fraction that follows
+    from it (work / time / peak) and the bytes moved per call.  None when the file or its last line is missing."""
+    import re
+    path = os.path.join(ROOT, "profiles", PROFILE_FILE.get(name, ""))
+    try:
+        with open(path) as f:
+            m = re.search(r"^bench\.py reads: (.*)$", f.read(), re.M)
+    except OSError:
+        return None
+    if not m:
+        return None
+    kv = dict(t.split("=") for t in m.group(1).split())
+    us = float(kv["kernel_us"])
+    out = {"file": "profiles/" + PROFILE_FILE[name], "kernel_us": us, "frac": round(work / (us * 1e-6) / peak, 4)}
+    if "fetch_bytes" in kv and "write_bytes" in kv:
+        out["traffic"] = float(kv["fetch_bytes"]) + float(kv["write_bytes"])
+    return out
+
+
+def attach_profile(roof, name, work=None):
+    """roofline.profile / roofline.traffic of a workload from its committed profile (work in flop or bytes, as the bound says)."""
+    work = roof["work_per_launch"] if work is None else work
+    peak = roof["peak"] * (1e12 if roof["bound"] == "mfma" else 1e9)
+    prof = profile_figures(name, work, peak)
+    roof["profile"] = prof
+    roof["traffic"] = prof.get("traffic") if prof else None
 
 SECONDARY = ("c1", "c3", "c4_dedx", "c4_dedw", "c5", "cast_fp8_143", "cast_bf16", "dequant_fp8_143")
 
@@ -74,7 +111,7 @@ class Bench:
         self.threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
         self._ref = self._orc = None
 
-    def settle(self, fn, seconds=0.06):
+    def settle(self, fn, seconds=SETTLE_MS * 1e-3):
         """Calls fn back to back for some tens of milliseconds.  After an idle period (operand set-up on the host) the device
         needs about 50 ms of work to reach the rate it then sustains: the headline GEMM takes 63-74 us per call over the first
         25 ms, 61 us up to 45 ms, and 59.7-59.9 us from there on for as long as it was watched (2.5 s).  Every measurement here
@@ -100,6 +137,45 @@ class Bench:
         e1.record(self.stream)
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / n * 1e-3
+
+    def per_launch(self, fn, n=60, group=5):
+        """Distribution of the stream time per call over n x group consecutive calls of fn (n >= 50 intervals): an event after
+        every `group` calls, each interval divided by `group`.  An event is a marker on the stream and costs about 3.5 us
+        of stream time itself (one per interval, so 0.7 us per call at group = 5): the figures of this pass sit that much above
+        the mean of the marker-free timed region, which stays the reported one; `marker_us_per_call` says how much."""
+        torch = self.torch
+        n = max(n, 50)
+        self.settle(fn)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(self.stream)
+        for _ in range(n * group):
+            fn()
+        e1.record(self.stream)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+        ev[0].record(self.stream)
+        for i in range(n):
+            for _ in range(group):
+                fn()
+            ev[i + 1].record(self.stream)
+        torch.cuda.synchronize()
+        free = e0.elapsed_time(e1) * 1e3 / (n * group)
+        us = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 / group for i in range(n))
+        med = us[n // 2] if n % 2 else 0.5 * (us[n // 2 - 1] + us[n // 2])
+        mean = sum(us) / n
+        return {"launches": n * group, "intervals": n, "calls_per_interval": group, "mean": round(mean, 3), "median": round(med, 3), "min": round(us[0], 3),
+                "max": round(us[-1], 3), "mean_without_markers": round(free, 3), "marker_us_per_call": round(mean - free, 3)}
+
+    def rotating(self, fns, n=60):
+        """The same call on len(fns) separate sets of operands and outputs taken in turn, which together hold more than the
+        memory-side cache: no call finds its operands, or the lines of its output, where its predecessor on the same set left
+        them.  Returns (mean seconds per call, per-launch distribution)."""
+        k = [0]
+
+        def step():
+            fns[k[0] % len(fns)]()
+            k[0] += 1
+
+        return self.timed(step, n=max(n, 4 * len(fns))), self.per_launch(step, n=n)
 
     def clocked(self, fn, n=30):
         """The shader clock the large-tile kernels ran at during n back-to-back calls of fn, and how long a workgroup took
@@ -186,13 +262,25 @@ class Bench:
 def mfma_roofline(flop, seconds, kind, kernel):
     achieved = flop / seconds / 1e12
     return {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS[kind], "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS[kind], 4),
-            "traffic": None, "kernel": kernel, "kernel_ms": round(seconds * 1e3, 5)}
+            "traffic": None, "kernel": kernel, "kernel_ms": round(seconds * 1e3, 5), "settle_ms": SETTLE_MS, "work_per_launch": flop}
+
+
+def rotating_figures(b, fns, work, roof, set_bytes):
+    """roofline.rotating: the workload's call cycling through len(fns) operand / output sets (b.rotating)."""
+    t, dist = b.rotating(fns)
+    scale = 1e12 if roof["bound"] == "mfma" else 1e9
+    return {"sets": len(fns), "bytes_cycled": int(set_bytes * len(fns)), "kernel_ms": round(t * 1e3, 5), "achieved": round(work / t / scale, 2),
+            "frac": round(work / t / scale / roof["peak"], 4), "per_launch_us": dist}
+
+
+def n_sets(set_bytes):
+    return max(2, -(-ROTATE_BYTES // int(set_bytes)))
 
 
 def hbm_roofline(nbytes, seconds, kernel):
     achieved = nbytes / seconds / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4),
-            "traffic": None, "kernel": kernel, "kernel_ms": round(seconds * 1e3, 5)}
+            "traffic": None, "kernel": kernel, "kernel_ms": round(seconds * 1e3, 5), "settle_ms": SETTLE_MS, "work_per_launch": nbytes}
 
 
 # ---- the headline workload: configs[1] -------------------------------------------------------------------------------------------
@@ -260,14 +348,25 @@ def run_c2(b):
                                "output (BASELINE.json configs[1]); library default policy for fp8 special codes", "op": "ab", "M": M, "N": N, "K": K,
                    "scale_exp_a": eA, "scale_exp_b": eB},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["fp8"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS["fp8"], 4), "traffic": GEMM_TRAFFIC_BYTES,
-                     "kernel": "gemm_fp8_w4_kernel<0, false, true>", "kernel_ms": round(kernel_ms, 5),
+                     "frac": round(achieved / PEAK_TFLOPS["fp8"], 4), "traffic": None,
+                     "kernel": "gemm_fp8_w4_kernel<0, false, true>", "kernel_ms": round(kernel_ms, 5), "settle_ms": SETTLE_MS, "work_per_launch": flop,
                      "policy": "check (default): the workgroups inspect the operand bytes they multiply and share what they find per operand panel; a tile whose panels hold a special code is computed again, exactly, inside the same launch",
                      "assume_none": {"achieved": round(assumed, 2), "frac": round(assumed / PEAK_TFLOPS["fp8"], 4), "kernel_ms": round(assumed_s * 1e3, 5),
                                      "kernel": "gemm_fp8_w4_kernel<0, false, false>",
                                      "policy": "the caller promises operands without exponent-all-ones codes (they come out of the saturating quantiser)"}},
     }
 
+    attach_profile(result["roofline"], "c2", flop)
+    # every launch on its own (events between the calls), and the same call cycling through operand / output sets that
+    # together exceed the memory-side cache
+    result["roofline"]["per_launch_us"] = b.per_launch(step, n=60)
+    set_bytes = 2 * M * K + 2 * M * N
+    sets = [(qa, qb, out)] + [(qa.clone(), qb.clone(), torch.zeros_like(out)) for _ in range(n_sets(set_bytes) - 1)]
+    descs = [(MmeSimTensor([N, M], 2, abi.BF16, o), MmeSimTensor([K, M], 2, abi.FP8_143, a, 7), MmeSimTensor([N, K], 2, abi.FP8_143, w, 7)) for a, w, o in sets]
+    fns = [(lambda y=y, x=x, w=w: calc.doBatchGemm(y, x, w, abi.OP_AB, epilogue=epi)) for y, x, w in descs]
+    result["roofline"]["rotating"] = rotating_figures(b, fns, flop, result["roofline"], set_bytes)
+    del sets, descs, fns
+    torch.cuda.empty_cache()
     # the clock the kernel ran at (all-zero operands would let the device hold 2400 MHz; these operands do not), and what
     # bare matrix instructions sustain on zero and on random operands
     result["roofline"]["clock"] = b.clocked(step, n=50)
@@ -328,6 +427,7 @@ def run_c1(b):
     flop = 2.0 * n ** 3
     res = {"workload": "bf16 GEMM 512^3 -> fp32 (configs[0])", "value": round(flop / t / 1e12, 2), "unit": "TFLOP/s",
            "roofline": mfma_roofline(flop, t, "bf16", "gemm_2byte_fast128_kernel")}
+    res["roofline"]["per_launch_us"] = b.per_launch(lambda: calc.doBatchGemm(Y1, A1, B1, abi.OP_AB))
     res["roofline"]["clock"] = b.clocked(lambda: calc.doBatchGemm(Y1, A1, B1, abi.OP_AB))
     if b.cpu:
         want = np.zeros(n * n, np.float32)
@@ -362,6 +462,13 @@ def run_c3(b):
     nbytes = 2.0 * (np.prod(xs) + np.prod(ws) + np.prod(ys))
     roof = mfma_roofline(flop, t, "bf16", "conv_fwd_resident_kernel<56>")
     roof["hbm_GB/s_algorithmic"] = round(nbytes / t / 1e9, 1)  # (288 flop per byte: within 10 % of the ridge)
+    roof["per_launch_us"] = b.per_launch(lambda: calc.doConvolution(YT, XT, WT, YT, cp, abi.OP_FWD, epilogue=e))
+    set_bytes = 2 * (tx.numel() + tw.numel() + ty.numel())
+    sets = [(MmeSimTensor(xs, 5, abi.BF16, tx.clone()), MmeSimTensor(ws, 5, abi.BF16, tw.clone()), MmeSimTensor(ys, 5, abi.BF16, torch.zeros_like(ty)))
+            for _ in range(n_sets(set_bytes) - 1)] + [(XT, WT, YT)]
+    roof["rotating"] = rotating_figures(b, [(lambda x_=x_, w_=w_, y_=y_: calc.doConvolution(y_, x_, w_, y_, cp, abi.OP_FWD, epilogue=e)) for x_, w_, y_ in sets],
+                                        flop, roof, set_bytes)
+    del sets
     res = {"workload": "bf16 conv2d fwd N=64 56x56 C=K=64 3x3 s1 p1, fused bf16 output (configs[2])", "value": round(flop / t / 1e12, 2),
            "unit": "TFLOP/s", "roofline": roof}
     if b.cpu:
@@ -412,6 +519,13 @@ def _run_c4(b, op):
     kernel = "conv_2byte_fast128_kernel" if op == abi.OP_DEDX else "conv_dedw_2byte_fast128_kernel + splitk_reduce_kernel"
     res = {"workload": "bf16 conv2d %s N=32 28x28 C=K=256 3x3 s1 p1, fp32 output (configs[3])" % name, "value": round(flop / t / 1e12, 2),
            "unit": "TFLOP/s", "roofline": mfma_roofline(flop, t, "bf16", kernel)}
+    res["roofline"]["per_launch_us"] = b.per_launch(lambda: calc.doConvolution(OT, XT, WT, YT, cp, op))
+    set_bytes = 2 * (XT.data().numel() + WT.data().numel() + YT.data().numel()) + 4 * to.numel()
+    sets = [(MmeSimTensor(xs, 5, abi.BF16, XT.data().clone()), MmeSimTensor(ws, 5, abi.BF16, WT.data().clone()), MmeSimTensor(ys, 5, abi.BF16, YT.data().clone()),
+             MmeSimTensor(osz, 5, abi.FP32, torch.zeros_like(to))) for _ in range(n_sets(set_bytes) - 1)] + [(XT, WT, YT, OT)]
+    res["roofline"]["rotating"] = rotating_figures(b, [(lambda x_=x_, w_=w_, y_=y_, o_=o_: calc.doConvolution(o_, x_, w_, y_, cp, op)) for x_, w_, y_, o_ in sets],
+                                                   flop, res["roofline"], set_bytes)
+    del sets
     res["roofline"]["clock"] = b.clocked(lambda: calc.doConvolution(OT, XT, WT, YT, cp, op))
     if op == abi.OP_DEDX:
         res["roofline"]["matrix_core_ceiling"] = b.matrix_core_ceiling(abi.BF16)
@@ -479,11 +593,16 @@ def run_c5(b):
                        "scales, fp8_143 output (configs[4]); library default policy for fp8 special codes", "value": round(flop / t / 1e12, 2),
            "unit": "TFLOP/s", "roofline": mfma_roofline(flop, t, "fp8", "gemm_fp8_persistent_chk_kernel<2, false>"),
            "scale_exp": {"a": sa, "out": so, "b_per_channel_min_max": [int(sb.min()), int(sb.max())]}}
+    res["roofline"]["per_launch_us"] = b.per_launch(lambda: calc.doBatchGemm(Y5, A5, B5, abi.OP_AB, epilogue=e5), n=50, group=2)
     res["roofline"]["clock"] = b.clocked(lambda: calc.doBatchGemm(Y5, A5, B5, abi.OP_AB, epilogue=e5), n=10)
     if b.cpu:
         orc = b.oracle_lib()
+        # 64 rows drawn at random over all four batch elements (16 of each): rows in the middle of the walk over the tiles
         r = 64
-        a8 = qa[:r * K5].cpu().numpy()
+        prng = np.random.default_rng(55)
+        rows = np.sort(np.concatenate([bz * M5 + prng.choice(M5, r // b5, replace=False) for bz in range(b5)]))
+        ridx = torch.from_numpy(rows).cuda()
+        a8 = qa.view(b5 * M5, K5)[ridx].cpu().numpy().ravel()
         b8 = qb.cpu().numpy()
         colh = col.cpu().numpy().astype(np.int32)
         acc = np.zeros(r * N5, np.float32)
@@ -492,13 +611,14 @@ def run_c5(b):
         cpu_s, kind = b.cpu_gemm(do, da, db, abi.OP_AB)
         want = np.zeros(r * N5, np.uint8)
         assert orc.orc_cast_from_fp32(want.ctypes.data, abi.FP8_143, 7, 0, acc.ctypes.data, r * N5, so - sa, colh.ctypes.data, N5, 0, 0, 1, 0, 0) == 0
-        got = o5[:r * N5].cpu().numpy()
+        got = o5.view(b5 * M5, N5)[ridx].cpu().numpy().ravel()
         dec = lambda c: _decode_fp8_143_b7(c)
         wf, gf = dec(want), dec(got)
-        res["parity"] = {"rows_checked": r, "rel_frobenius_vs_reference_fp8": float(np.linalg.norm(gf - wf) / np.linalg.norm(wf)),
+        res["parity"] = {"rows_checked": r, "rows": "16 rows drawn at random from each of the 4 batch elements",
+                         "rel_frobenius_vs_reference_fp8": float(np.linalg.norm(gf - wf) / np.linalg.norm(wf)),
                          "fp8_codes_equal_frac": float(np.mean(got == want)), "nonzero_codes_frac": float(np.mean((want & 0x7F) != 0)), "tolerance": 1e-2}
         res["cpu_baseline"] = {"value": round(2.0 * r * N5 * K5 / cpu_s / 1e12, 7), "unit": "TFLOP/s", "cores": b.threads, "kind": kind,
-                               "sample": "first %d rows of batch 0 against the full B (%.2f GFLOP of the 962 GFLOP job, doBatchGemm only), %.1f s wall"
+                               "sample": "%d rows drawn from all four batch elements against the full B (%.2f GFLOP of the 962 GFLOP job, doBatchGemm only), %.1f s wall"
                                          % (r, 2.0 * r * N5 * K5 / 1e9, cpu_s)}
     return res
 
@@ -599,7 +719,7 @@ def main():
             print("unknown workload %r" % args.only, file=sys.stderr)
             sys.exit(2)
         res = WORKLOADS[args.only](b)
-        res["roofline"]["traffic"] = TRAFFIC_BYTES.get(args.only)
+        attach_profile(res["roofline"], args.only)
         print(json.dumps({args.only: res}))
         b.calc.close()
         return
@@ -608,7 +728,7 @@ def main():
         result["secondary"] = {}
         for name in SECONDARY:
             result["secondary"][name] = WORKLOADS[name](b)
-            result["secondary"][name]["roofline"]["traffic"] = TRAFFIC_BYTES.get(name)
+            attach_profile(result["secondary"][name]["roofline"], name)
             b.torch.cuda.empty_cache()
     if args.extra:
         result["extra"] = extra_measurements(b.calc, b.stream)

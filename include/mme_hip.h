@@ -160,6 +160,12 @@ typedef struct mme_hip_conv_params
  * harness in between, done in registers instead of through an fp32 tensor:
  *     y = cast( relu?( acc * 2^scale_exp * 2^col_scale_exp[n] ) )
  * Each multiplication is an fp32 multiplication by an exact power of two.
+ * With a stochastic rounding mode (4, 7) the conversion is the one of doActivation,
+ * which runs over the output tensor's whole span in memory
+ * (mme_reference_impl.cpp:1155, sim_tensor_base.cpp:177-194): the bytes between the
+ * rows of an output with strided rows are then overwritten with the code of zero,
+ * as they are when the reference converts a fresh accumulator tensor of that shape.
+ * The other rounding modes leave those bytes untouched.
  */
 typedef struct mme_hip_epilogue
 {
@@ -395,7 +401,14 @@ int mme_hip_batch_gemm_dev(mme_hip_handle          h,
  * in mme_hip_last_error (large fp8 operands in an inf/NaN mode the hardware formats lack need decoded copies for the
  * fall-back: set MME_HIP_FP8_SPECIALS_ASSUME_NONE where that holds, or use mme_hip_batch_gemm_dev).  All handles of a
  * device share that device's array: calls that overlap in time on one device race on it, so serialise them (one stream,
- * or events between streams).
+ * or events between streams).  A stochastic rounding mode in the epilogue is served too (the LFSR jump table exists since
+ * mme_hip_create; the fp32 intermediate comes out of the same array).
+ *
+ * Recording the other device-pointer entry points into a HIP graph: the recorded launches hold the addresses of the handle's
+ * grow-only work spaces.  A work space must have its size before the recording starts (growing one on a recording stream
+ * fails with the HIP error and leaves it as it was); once a handle has seen a recording stream it keeps every block it
+ * outgrows until mme_hip_destroy instead of freeing it, so later larger calls do not invalidate a graph.  Destroy the graph
+ * before the handle.
  */
 #define MME_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
 int mme_hip_batch_gemm_dev_noalloc(mme_hip_handle          h,

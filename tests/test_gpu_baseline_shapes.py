@@ -140,8 +140,10 @@ def test_c4_conv_dedx_dedw_full_size(calc, orc):
 
 def test_c5_batched_mixed_fp8_gemm_full_size(calc, orc):
     """Batched fp8 GEMM 4 x (2048 x 4096) x (4096 x 14336): A fp8_143 (bias 7), B fp8_152 (bias 15) shared by the batch,
-    per-column power-of-two descale, fp8_143 output with saturation.  A slab of 16 rows in two batch elements against the
-    oracle (accumulate, descale, cast): codes may differ by one where the accumulators straddle a rounding boundary."""
+    per-column power-of-two descale, fp8_143 output with saturation.  Slabs of 16 rows in all four batch elements against the
+    oracle (accumulate, descale, cast): the first and the last tile row of the job, and tile rows in the middle of the walk
+    over the tiles (batch elements 1 and 2, slabs that start inside a tile and one that straddles two tile rows).  Codes may
+    differ by one where the accumulators straddle a rounding boundary."""
     import torch
     rng = np.random.default_rng(3)
     b5, M, K, N = 4, 2048, 4096, 14336
@@ -164,7 +166,7 @@ def test_c5_batched_mixed_fp8_gemm_full_size(calc, orc):
     calc.synchronize()
     got = out.cpu().numpy().reshape(b5, M, N)
     rows = 16
-    for b, r0 in ((0, 0), (3, M - rows)):
+    for b, r0 in ((0, 0), (1, 3 * 256 + 40), (2, 5 * 256 - 8), (2, 1024 + 117), (3, M - rows)):
         slab = np.ascontiguousarray(qa[b, r0:r0 + rows].reshape(-1))
         acc = np.zeros(rows * N, np.float32)
         da, db, do = desc(slab, [K, rows], abi.FP8_143, 7), desc(qb.reshape(-1), [N, K], abi.FP8_152, 15), desc(acc, [N, rows], abi.FP32)

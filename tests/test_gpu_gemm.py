@@ -471,7 +471,9 @@ def test_fused_epilogue_with_stochastic_rounding(orc, out_dt, out_bias, rm, M, N
             b = random_operand(rng, abi.FP8_152, N * K, orc, 15, scale=0.05)
             X = MmeSimTensor([K, M], 2, abi.FP8_143, torch.from_numpy(a).cuda(), 7)
             W = MmeSimTensor([N, K], 2, abi.FP8_152, torch.from_numpy(b).cuda(), 15)
-            out = torch.zeros(M * ld, dtype=td, device="cuda")
+            # (a sentinel in every byte: with a stochastic mode the gaps between strided rows are converted too and must come
+            # out as the code of zero, as the reference's doActivation over the tensor's span leaves them)
+            out = torch.full((M * ld,), 0x55, dtype=td, device="cuda")
             epi = Epilogue(scale_exp=-1, col_scale_exp=torch.from_numpy(col).cuda(), relu=bool(call), rm=rm, clipFp=True)
             fused_calc.doBatchGemm(MmeSimTensor([N, M], 2, out_dt, out, out_bias, strides=so), X, W, abi.OP_AB, epilogue=epi)
             fused_calc.synchronize()
@@ -605,6 +607,45 @@ def test_fp8_fast_kernel_epilogue_overflow_takes_exact_conversion(calc, orc, cli
     got = out.cpu().numpy().view(np.uint16)
     assert np.array_equal(got, want)
     assert (np.any((want & 0x7FFF) == 0x7F7F) if clip else np.any((want & 0x7FFF) == 0x7F80))
+
+
+@pytest.mark.parametrize("policy", [abi.FP8_SPECIALS_CHECK, abi.FP8_SPECIALS_ASSUME_NONE])
+@pytest.mark.parametrize("clip", [False, True])
+@pytest.mark.parametrize("scale_exp", [84, 88, 92])
+def test_fp8_152_operands_of_largest_magnitude_with_a_large_descale(calc, orc, scale_exp, clip, policy):
+    """fp8_152 x fp8_152 with every operand at the largest finite magnitude (57344, about 2^15.8): products reach 2^31.6 and
+    sums over K = 4096 2^43.6, so a power-of-two factor of 2^84 and more takes them beyond the fp32 and bf16 ranges.  The
+    host may then neither promise the epilogue finite values nor hand the factor to the matrix instruction: the fused bf16
+    output must equal the oracle's cast of the GPU's own fp32 accumulators, bit for bit, under both policies for special codes."""
+    import torch
+    M, N, K = 256, 256, 4096
+    rng = np.random.default_rng(scale_exp)
+    a = np.where(rng.random(M * K) < 0.5, 0x7B, 0xFB).astype(np.uint8)
+    b = np.full(N * K, 0x7B, np.uint8)
+    # rows whose signs cancel down to a finite result, rows that do not
+    a.reshape(M, K)[::3] = 0x7B
+    ta, tb = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    X, W = MmeSimTensor([K, M], 2, abi.FP8_152, ta, 15), MmeSimTensor([N, K], 2, abi.FP8_152, tb, 15)
+    acc = torch.zeros(M * N, dtype=torch.float32, device="cuda")
+    out = torch.zeros(M * N, dtype=torch.int16, device="cuda")
+    calc.setFp8SpecialsPolicy(policy)
+    try:
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.FP32, acc), X, W, abi.OP_AB)
+        calc.doBatchGemm(MmeSimTensor([N, M], 2, abi.BF16, out), X, W, abi.OP_AB, epilogue=Epilogue(scale_exp=scale_exp, clipFp=clip))
+        assert calc.lastContractionForm()["large_tile"]
+        calc.synchronize()
+    finally:
+        calc.setFp8SpecialsPolicy(abi.FP8_SPECIALS_CHECK)
+    acc_h = acc.cpu().numpy()
+    assert np.isfinite(acc_h).all() and np.abs(acc_h).max() == np.float32(57344.0 * 57344.0 * K)
+    want = np.zeros(M * N, np.uint16)
+    assert orc.orc_cast_from_fp32(want.ctypes.data, abi.BF16, 0, 0, acc_h.ctypes.data, M * N, scale_exp, None, 0, 0, 0, int(clip), 0, 0) == 0
+    got = out.cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, want), int(np.argmax(got != want))
+    # (2^84 leaves the largest sum, 49 * 2^122, just inside the bf16 range; 2^88 and 2^92 do not)
+    # (there the product with the factor is already infinite in fp32, which clipFp alone leaves infinite)
+    assert scale_exp < 85 or np.any((want & 0x7FFF) == 0x7F80)
+    assert np.any((want & 0x7FFF) < 0x7F00)  # rows whose signs cancel stay finite
 
 
 @pytest.mark.parametrize("clip", [False, True])

@@ -94,7 +94,26 @@ def test_fp8_one_round_gemm_recorded_into_a_graph_settles_special_codes_on_every
                 assert np.array_equal(np.isnan(g), np.isnan(ref)) and np.array_equal(np.isinf(g), np.isinf(ref)), (step, which)
                 f = np.isfinite(ref)
                 assert np.array_equal(g[~f & ~np.isnan(ref)], ref[~f & ~np.isnan(ref)]) and rel_frobenius(g[f], ref[f]) <= 1e-4, (step, which)
-        del graph
+        # a larger direct call on the same handle outgrows the work space that the recorded fall-back launches point into (the
+        # decoded copies of three batch elements of A): the handle has seen a recording stream, so it keeps the old block,
+        # and a replay that meets a special code still computes the right thing
+        ta3, out3 = torch.cat([ta, ta, ta]), torch.zeros(3 * M * N, dtype=torch.float32, device="cuda")
+        c.doBatchGemm(MmeSimTensor([N, M, 3, 1, 1], 5, abi.FP32, out3), MmeSimTensor([K, M, 3, 1, 1], 5, abi.FP8_143, ta3, 7),
+                      MmeSimTensor([N, K, 1, 1, 1], 5, abi.FP8_143, tb, 7), abi.OP_AB)
+        c.synchronize()
+        del ta3, out3
+        spare = [torch.full((1 << 22,), 1.5, dtype=torch.float32, device="cuda") for _ in range(8)]  # would land in a freed block
+        a = a0.copy()
+        a[5, 9] = 0x78
+        ta.copy_(torch.from_numpy(a.ravel()))
+        tb.copy_(torch.from_numpy(b0.ravel()))
+        torch.cuda.synchronize()
+        got, want = replayed(), direct()
+        assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+        fin = np.isfinite(want)
+        assert not fin.all() and rel_frobenius(got[fin], want[fin]) <= 1e-4
+        assert all(float(t.min()) == 1.5 and float(t.max()) == 1.5 for t in spare)
+        del graph, spare
     finally:
         c.setStream(None)
         c.close()

@@ -101,3 +101,64 @@ def test_no_alloc_entry_point_equals_the_allocating_one():
         assert lib.mme_hip_synchronize(h) == 0
     finally:
         lib.mme_hip_destroy(h)
+
+
+def test_no_alloc_entry_point_first_on_a_fresh_handle():
+    """A handle whose very first calls go through the entry point that allocates nothing: split-k bf16, fp8 operands with an
+    inf code (flag cell and decoded copies), fp32 operands (three bf16 parts) and a fused epilogue with stochastic rounding
+    (the LFSR jump table must exist since mme_hip_create).  The free device memory does not move across those calls, and
+    the outputs equal those of a second handle that takes the allocating entry point (which also runs first, so that the
+    code objects are loaded and torch's allocator holds its blocks before free memory is read)."""
+    import torch
+    lib = abi.load_library()
+    rng = np.random.default_rng(43)
+
+    def operands(dt, M, N, K):
+        if dt == abi.BF16:
+            return (torch.from_numpy(_bf16(rng.standard_normal(M * K)).view(np.int16)).cuda(), torch.from_numpy(_bf16(rng.standard_normal(K * N)).view(np.int16)).cuda())
+        if dt == abi.FP32:
+            return (torch.from_numpy(rng.standard_normal(M * K).astype(np.float32)).cuda(), torch.from_numpy(rng.standard_normal(K * N).astype(np.float32)).cuda())
+        ca = rng.integers(0, 0x60, M * K).astype(np.uint8) | (rng.integers(0, 2, M * K).astype(np.uint8) << 7)
+        cb = rng.integers(0, 0x60, K * N).astype(np.uint8) | (rng.integers(0, 2, K * N).astype(np.uint8) << 7)
+        return torch.from_numpy(ca).cuda(), torch.from_numpy(cb).cuda()
+
+    # (name, dtype, bias, M, N, K, output type, rounding mode of the fused epilogue or None, code to plant in A)
+    cases = [("bf16 split-k", abi.BF16, 0, 256, 256, 8192, abi.FP32, None, None),
+             ("fp8 with inf", abi.FP8_143, 7, 512, 256, 1024, abi.FP32, None, 0x78),
+             ("fp32 three parts", abi.FP32, 0, 256, 256, 1024, abi.FP32, None, None),
+             ("fp8 stochastic epilogue", abi.FP8_143, 7, 256, 256, 512, abi.BF16, 4, None)]
+    data = []
+    for name, dt, bias, M, N, K, out_dt, rm, plant in cases:
+        a, b = operands(dt, M, N, K)
+        if plant is not None:
+            a[11 * K + 5] = plant
+        tdt = torch.float32 if out_dt == abi.FP32 else torch.int16
+        epi = None
+        if rm is not None:
+            epi = abi.Epilogue()
+            epi.scale_exp = -3
+            epi.rounding_mode = rm
+            epi.clip_fp = 1
+        data.append((name, dt, bias, M, N, K, out_dt, epi, a, b, torch.full((M * N,), 7, dtype=tdt, device="cuda"), torch.full((M * N,), 9, dtype=tdt, device="cuda")))
+    h_alloc = _handle(lib)
+    try:
+        for name, dt, bias, M, N, K, out_dt, epi, a, b, o1, o2 in data:
+            assert _run(lib, h_alloc, lib.mme_hip_batch_gemm_dev, a, b, o1, [K, M], [N, K], [N, M], dt, bias, 0, out_dt, abi.OP_AB, epi) == 0, lib.mme_hip_last_error(h_alloc)
+        assert lib.mme_hip_synchronize(h_alloc) == 0
+        h = _handle(lib)
+        try:
+            torch.cuda.synchronize()
+            free0 = torch.cuda.mem_get_info()[0]
+            for name, dt, bias, M, N, K, out_dt, epi, a, b, o1, o2 in data:
+                print("no-alloc first on a fresh handle:", name, flush=True)
+                assert _run(lib, h, lib.mme_hip_batch_gemm_dev_noalloc, a, b, o2, [K, M], [N, K], [N, M], dt, bias, 0, out_dt, abi.OP_AB, epi) == 0, lib.mme_hip_last_error(h)
+                assert lib.mme_hip_synchronize(h) == 0
+            assert torch.cuda.mem_get_info()[0] == free0
+            for name, dt, bias, M, N, K, out_dt, epi, a, b, o1, o2 in data:
+                r1, r2 = o1.cpu().numpy(), o2.cpu().numpy()
+                assert np.array_equal(r1.view(np.uint8), r2.view(np.uint8)), name
+                assert np.any(r1 != 7), name
+        finally:
+            lib.mme_hip_destroy(h)
+    finally:
+        lib.mme_hip_destroy(h_alloc)
