@@ -139,6 +139,11 @@ class Bench:
         return e0.elapsed_time(e1) / n * 1e-3
 
     def per_launch(self, fn, n=60, group=5):
+        if self.args.plain:
+            return None
+        return self._per_launch(fn, n, group)
+
+    def _per_launch(self, fn, n=60, group=5):
         """Distribution of the stream time per call over n x group consecutive calls of fn (n >= 50 intervals): an event after
         every `group` calls, each interval divided by `group`.  An event is a marker on the stream and costs about 3.5 us
         of stream time itself (one per interval, so 0.7 us per call at group = 5): the figures of this pass sit that much above
@@ -175,9 +180,14 @@ class Bench:
             fns[k[0] % len(fns)]()
             k[0] += 1
 
-        return self.timed(step, n=max(n, 4 * len(fns))), self.per_launch(step, n=n)
+        return self.timed(step, n=max(n, 4 * len(fns))), self._per_launch(step, n=n)
 
     def clocked(self, fn, n=30):
+        if self.args.plain:
+            return None
+        return self._clocked(fn, n)
+
+    def _clocked(self, fn, n=30):
         """The shader clock the large-tile kernels ran at during n back-to-back calls of fn, and how long a workgroup took
         (stamps taken inside the kernels; the published peak rates are quoted at 2400 MHz).  call_us_with_probe is the wall
         time per call while the stamps are on, the read-out of the stamps at the end included (2 us per call at n = 50): the
@@ -200,6 +210,8 @@ class Bench:
         """What back-to-back matrix instructions with operands in registers sustain on this device: with all-zero operands
         (the published rate) and with operands that change from instruction to instruction (power management lowers the clock)."""
         out = {}
+        if self.args.plain:
+            return None
         for name, rnd in (("zero_operands", 0), ("random_operands", 1)):
             tf, mhz = self.calc.matrixCoreRate(dtype, rnd, iters=4096, launches=10)
             out[name] = {"TFLOP/s": round(tf, 1), "shader_clock_mhz": round(mhz)}
@@ -267,6 +279,8 @@ def mfma_roofline(flop, seconds, kind, kernel):
 
 def rotating_figures(b, fns, work, roof, set_bytes):
     """roofline.rotating: the workload's call cycling through len(fns) operand / output sets (b.rotating)."""
+    if b.args.plain:
+        return None
     t, dist = b.rotating(fns)
     scale = 1e12 if roof["bound"] == "mfma" else 1e9
     return {"sets": len(fns), "bytes_cycled": int(set_bytes * len(fns)), "kernel_ms": round(t * 1e3, 5), "achieved": round(work / t / scale, 2),
@@ -361,7 +375,7 @@ def run_c2(b):
     # together exceed the memory-side cache
     result["roofline"]["per_launch_us"] = b.per_launch(step, n=60)
     set_bytes = 2 * M * K + 2 * M * N
-    sets = [(qa, qb, out)] + [(qa.clone(), qb.clone(), torch.zeros_like(out)) for _ in range(n_sets(set_bytes) - 1)]
+    sets = [(qa, qb, out)] + [(qa.clone(), qb.clone(), torch.zeros_like(out)) for _ in range(0 if args.plain else n_sets(set_bytes) - 1)]
     descs = [(MmeSimTensor([N, M], 2, abi.BF16, o), MmeSimTensor([K, M], 2, abi.FP8_143, a, 7), MmeSimTensor([N, K], 2, abi.FP8_143, w, 7)) for a, w, o in sets]
     fns = [(lambda y=y, x=x, w=w: calc.doBatchGemm(y, x, w, abi.OP_AB, epilogue=epi)) for y, x, w in descs]
     result["roofline"]["rotating"] = rotating_figures(b, fns, flop, result["roofline"], set_bytes)
@@ -465,7 +479,7 @@ def run_c3(b):
     roof["per_launch_us"] = b.per_launch(lambda: calc.doConvolution(YT, XT, WT, YT, cp, abi.OP_FWD, epilogue=e))
     set_bytes = 2 * (tx.numel() + tw.numel() + ty.numel())
     sets = [(MmeSimTensor(xs, 5, abi.BF16, tx.clone()), MmeSimTensor(ws, 5, abi.BF16, tw.clone()), MmeSimTensor(ys, 5, abi.BF16, torch.zeros_like(ty)))
-            for _ in range(n_sets(set_bytes) - 1)] + [(XT, WT, YT)]
+            for _ in range(0 if b.args.plain else n_sets(set_bytes) - 1)] + [(XT, WT, YT)]
     roof["rotating"] = rotating_figures(b, [(lambda x_=x_, w_=w_, y_=y_: calc.doConvolution(y_, x_, w_, y_, cp, abi.OP_FWD, epilogue=e)) for x_, w_, y_ in sets],
                                         flop, roof, set_bytes)
     del sets
@@ -522,7 +536,7 @@ def _run_c4(b, op):
     res["roofline"]["per_launch_us"] = b.per_launch(lambda: calc.doConvolution(OT, XT, WT, YT, cp, op))
     set_bytes = 2 * (XT.data().numel() + WT.data().numel() + YT.data().numel()) + 4 * to.numel()
     sets = [(MmeSimTensor(xs, 5, abi.BF16, XT.data().clone()), MmeSimTensor(ws, 5, abi.BF16, WT.data().clone()), MmeSimTensor(ys, 5, abi.BF16, YT.data().clone()),
-             MmeSimTensor(osz, 5, abi.FP32, torch.zeros_like(to))) for _ in range(n_sets(set_bytes) - 1)] + [(XT, WT, YT, OT)]
+             MmeSimTensor(osz, 5, abi.FP32, torch.zeros_like(to))) for _ in range(0 if b.args.plain else n_sets(set_bytes) - 1)] + [(XT, WT, YT, OT)]
     res["roofline"]["rotating"] = rotating_figures(b, [(lambda x_=x_, w_=w_, y_=y_, o_=o_: calc.doConvolution(o_, x_, w_, y_, cp, op)) for x_, w_, y_, o_ in sets],
                                                    flop, res["roofline"], set_bytes)
     del sets
@@ -656,6 +670,7 @@ def _run_cast(b, which):
         t = b.timed(lambda: calc.castToFp32(x, codes, abi.FP8_143, n, fpBias=7), n=20)
         res = {"workload": "fp8_143 (bias 7) -> fp32 dequantise, 2^28 elements", "value": round(n * 5 / t / 1e9, 1), "unit": "GB/s",
                "roofline": hbm_roofline(n * 5.0, t, "cast_to_fp32_kernel")}
+        res["roofline"]["per_launch_us"] = b.per_launch(lambda: calc.castToFp32(x, codes, abi.FP8_143, n, fpBias=7), n=50, group=2)
         if b.cpu:
             orc = b.oracle_lib()
             ch = codes[:ncpu].cpu().numpy()
@@ -674,6 +689,7 @@ def _run_cast(b, which):
     t = b.timed(lambda: calc.castFromFp32(o, dt, x, n, fpBias=7 if ob == 1 else 0, clipFp=True), n=20)
     res = {"workload": "%s cast, 2^28 elements of N(0,1) * 2^U[-12,12] with 2^-10 specials" % name, "value": round(n * (4 + ob) / t / 1e9, 1), "unit": "GB/s",
            "roofline": hbm_roofline(n * (4.0 + ob), t, kern)}
+    res["roofline"]["per_launch_us"] = b.per_launch(lambda: calc.castFromFp32(o, dt, x, n, fpBias=7 if ob == 1 else 0, clipFp=True), n=50, group=2)
     if b.cpu:
         xh = x[:ncpu].cpu().numpy()
         want = np.zeros(ncpu * ob, np.uint8)
@@ -701,6 +717,8 @@ def main():
     ap.add_argument("--no-secondary", action="store_true", help="time the headline workload only")
     ap.add_argument("--only", default=None, help="run one workload only (c2 or one of: %s), e.g. under a profiler" % ", ".join(SECONDARY))
     ap.add_argument("--cpu-rows", type=int, default=256, help="rows of A in the CPU baseline's M-slab")
+    ap.add_argument("--plain", action="store_true", help="the timed regions only: no per-call distribution, no rotating operand sets, no clock probe, no "
+                    "matrix-core ceiling (what the profiles under profiles/ are taken with, so that a traced average is the average of the timed calls)")
     ap.add_argument("--extra", action="store_true", help="also time further shapes and operand types (fp16 / ufp16 / fp32 GEMMs, fp8 convolutions, host-pointer calls)")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also launch a plain elementwise copy of 2^26 floats (256 MiB read, 256 MiB written) a few times: a "
