@@ -250,12 +250,27 @@ int mme_hip_set_wait_limit(mme_hip_handle h, unsigned polls);
  * device with nothing else to do, and the clock they held.
  *
  * mme_hip_last_contraction_form: which form of the contraction kernels the latest doBatchGemm / doConvolution call of this
- * handle launched: large_tile 1 when a large-tile kernel took it (0: the general kernel), the rows of its output tile (256 or
+ * handle launched: large_tile 1 when a large-tile kernel took it (0: the general kernel; 2: the forward kernel for 3 x 3
+ * filters over 64 -> 64 bf16 channels, whose other three figures are 0, 1, 8), the rows of its output tile (256 or
  * 128), the slices of the reduction (1: no split-k) and the wavefronts per workgroup (8, or 4 for the fp8 GEMM form with
  * 128 x 128 outputs per wavefront).  Lets a test state which kernel it is about.
+ *
+ * mme_hip_plan_batch_gemm / mme_hip_plan_convolution: the same four figures (form[0..3], in that order) for a call that is not
+ * made: what mme_hip_batch_gemm_dev / mme_hip_convolution_dev would launch for these descriptors on a device with num_cus
+ * compute units (<= 0: 256) under the given policy for fp8 special codes.  The call goes through the same checks and the same
+ * planning code as the real one, launches and allocates nothing and needs no device or handle; the data pointers of the
+ * descriptors are not dereferenced (their alignment matters: hand in the real ones, or any 16-byte aligned non-null value).
+ * Returns what the real call would return for a refused problem, with its message in `error` (may be NULL); form[0] is -1 for
+ * a problem that launches no contraction kernel (a zero-size common dimension).
  */
 int mme_hip_clock_probe(mme_hip_handle h, int enable);
 int mme_hip_last_contraction_form(mme_hip_handle h, int* large_tile, int* tile_rows, int* split_k, int* wavefronts);
+int mme_hip_plan_batch_gemm(const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, int op,
+                            const mme_hip_epilogue* epilogue, int num_cus, int fp8_specials_policy, int form[4], char* error,
+                            size_t error_bytes);
+int mme_hip_plan_convolution(const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, const mme_hip_tensor* y,
+                             const mme_hip_conv_params* params, int op, const mme_hip_epilogue* epilogue, int num_cus,
+                             int fp8_specials_policy, int form[4], char* error, size_t error_bytes);
 int mme_hip_clock_probe_read(mme_hip_handle h, double* shader_mhz, double* mean_us, double* max_us, int* workgroups);
 int mme_hip_matrix_core_rate(mme_hip_handle h, int dtype, int random_operands, int iters, int launches, double* tflops, double* shader_mhz);
 

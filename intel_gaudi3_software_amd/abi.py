@@ -140,6 +140,9 @@ def load_library():
     L.mme_hip_clock_probe.argtypes = [vp, C.c_int]
     L.mme_hip_clock_probe_read.argtypes = [vp, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int)]
     L.mme_hip_last_contraction_form.argtypes = [vp] + [C.POINTER(C.c_int)] * 4
+    L.mme_hip_plan_batch_gemm.argtypes = [_TP, _TP, _TP, C.c_int, C.POINTER(Epilogue), C.c_int, C.c_int, C.POINTER(C.c_int), C.c_char_p, C.c_size_t]
+    L.mme_hip_plan_convolution.argtypes = [_TP, _TP, _TP, _TP, C.POINTER(ConvParams), C.c_int, C.POINTER(Epilogue), C.c_int, C.c_int, C.POINTER(C.c_int),
+                                           C.c_char_p, C.c_size_t]
     L.mme_hip_matrix_core_rate.argtypes = [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
     L.mme_hip_set_fp8_specials_policy.argtypes = [vp, C.c_int]
     L.mme_hip_set_operand_clip.argtypes = [vp, C.c_int, C.c_int]
@@ -158,3 +161,29 @@ def load_library():
     L.mme_hip_absmax_dev.argtypes = [vp, vp, vp, C.c_size_t]
     _lib = L
     return L
+
+
+def _planned(rc, form, err):
+    if rc != 0:
+        raise ValueError("%s (status %d)" % (err.value.decode(), rc))
+    return {"large_tile": form[0], "tile_rows": form[1], "split_k": form[2], "wavefronts": form[3]}
+
+
+def plan_batch_gemm(out, x, w, op, epilogue=None, num_cus=256, fp8_specials_policy=FP8_SPECIALS_CHECK):
+    """Which kernel form ``mme_hip_batch_gemm_dev`` would launch for these descriptors (``mme_hip_plan_batch_gemm``): nothing
+    runs, no GPU is needed.  The descriptors' data pointers only matter through their alignment (``make_tensor(4096, ...)``
+    will do).  Raises ValueError with the library's message for a problem the real call would refuse."""
+    lib = load_library()
+    form, err = (C.c_int * 4)(), C.create_string_buffer(512)
+    rc = lib.mme_hip_plan_batch_gemm(C.byref(out), C.byref(x), C.byref(w), op, C.byref(epilogue) if epilogue is not None else None, num_cus,
+                                     fp8_specials_policy, form, err, 512)
+    return _planned(rc, form, err)
+
+
+def plan_convolution(out, x, w, y, params, op, epilogue=None, num_cus=256, fp8_specials_policy=FP8_SPECIALS_CHECK):
+    """The same for ``mme_hip_convolution_dev`` (``mme_hip_plan_convolution``)."""
+    lib = load_library()
+    form, err = (C.c_int * 4)(), C.create_string_buffer(512)
+    rc = lib.mme_hip_plan_convolution(C.byref(out), C.byref(x), C.byref(w), C.byref(y), C.byref(params), op,
+                                      C.byref(epilogue) if epilogue is not None else None, num_cus, fp8_specials_policy, form, err, 512)
+    return _planned(rc, form, err)

@@ -113,6 +113,9 @@ struct mme_hip_calc
     // has been; from then on the work spaces never free a block they outgrow (a graph may replay launches that point into it)
     bool                  recording = false;
     bool                  graph_seen = false;
+    // a handle without a device that only answers "which kernel form would this call launch" (mme_hip_plan_*): it goes
+    // through the same checks and the same planning as a real call, allocates nothing and skips every launch
+    bool                  dry_run = false;
     // diagnostics: per-workgroup clock stamps of the large-tile kernels (mme_hip_clock_probe), NULL while switched off
     DeviceBuffer          clock_probe_buf;
     uint64_t*             clock_probe = nullptr;
@@ -135,6 +138,13 @@ int fail(mme_hip_handle h, int code, const char* fmt, ...)
 
 int build_lfsr_jump(mme_hip_handle h);
 
+// a kernel launch of a contraction or conversion path: skipped by a planning handle (mme_hip_calc::dry_run)
+#define LAUNCH_TRY(h, expr)                  \
+    do                                       \
+    {                                        \
+        if (!(h)->dry_run) HIP_TRY(h, expr); \
+    } while (0)
+
 int hip_fail(mme_hip_handle h, hipError_t e, const char* what)
 {
     return fail(h, e == hipErrorOutOfMemory ? MME_HIP_ENOMEM : MME_HIP_EHIP, "%s: %s", what, hipGetErrorString(e));
@@ -151,6 +161,7 @@ int hip_fail(mme_hip_handle h, hipError_t e, const char* what)
 // read counts as recording: the careful side.)
 void note_recording(mme_hip_handle h)
 {
+    if (h->dry_run) return;
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(h->stream, &st) != hipSuccess)
     {
@@ -162,7 +173,7 @@ void note_recording(mme_hip_handle h)
 }
 
 // grows one of the handle's buffers (see DeviceBuffer)
-hipError_t grow(mme_hip_handle h, DeviceBuffer& buf, size_t bytes) { return buf.reserve(bytes, h->graph_seen); }
+hipError_t grow(mme_hip_handle h, DeviceBuffer& buf, size_t bytes) { return h->dry_run ? hipSuccess : buf.reserve(bytes, h->graph_seen); }
 
 // Work space of `bytes` for the current call: the handle's grow-only buffer `buf`, or, in a call that may not allocate, the
 // next piece of the device's static scratch array.
@@ -173,6 +184,11 @@ constexpr unsigned CHK_STATE_RING = 64;
 
 int take_ws(mme_hip_handle h, DeviceBuffer& buf, size_t bytes, void** out)
 {
+    if (h->dry_run)
+    {
+        *out = (void*) (uintptr_t) 4096; // (a planning handle never touches it; aligned and not null, like a real one)
+        return MME_HIP_OK;
+    }
     if (!h->noalloc)
     {
         HIP_TRY(h, grow(h, buf, bytes));
@@ -376,7 +392,7 @@ int next_flag_epoch(mme_hip_handle h, uint32_t** flag, uint32_t* epoch)
     if (!h->flag.p)
     {
         HIP_TRY(h, grow(h, h->flag, 256));
-        HIP_TRY(h, launch_fill_u32((uint32_t*) h->flag.p, 0u, 64, h->stream)); // epoch numbers start at 1
+        LAUNCH_TRY(h, launch_fill_u32((uint32_t*) h->flag.p, 0u, 64, h->stream)); // epoch numbers start at 1
     }
     *flag = (uint32_t*) h->flag.p;
     *epoch = ++h->specials_epoch;
@@ -517,7 +533,7 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
                 bstride[d] = view[i]->batch_stride[d] ? run : 0;
                 run *= eff[i][d];
             }
-            HIP_TRY(h, launch_split_bf16(dst, src[i], t[i]->dtype, a, h->stream));
+            LAUNCH_TRY(h, launch_split_bf16(dst, src[i], t[i]->dtype, a, h->stream));
             if (a.k_contig) set_plain_view(*v2[i], dst, (long long) kblocks * a.K, 1, true, 2, kblocks * a.K, bstride);
             else
                 set_plain_view(*v2[i], dst, 1, a.F, false, 2, a.F, bstride);
@@ -531,9 +547,9 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
     {
         float* d = i ? db : da;
         if (t[i]->dtype == MME_HIP_TF32)
-            HIP_TRY(h, launch_round_to_tf32(d, src[i], i ? nb : na, h->operand_clip_fp, h->operand_clip_inf_in, h->stream, flag, epoch));
+            LAUNCH_TRY(h, launch_round_to_tf32(d, src[i], i ? nb : na, h->operand_clip_fp, h->operand_clip_inf_in, h->stream, flag, epoch));
         else
-            HIP_TRY(h, launch_cast_to_fp32(d, src[i], t[i]->dtype, (int) t[i]->fp_bias, t[i]->inf_nan_mode, i ? nb : na, 1.0f, 0, nullptr, 0, h->stream,
+            LAUNCH_TRY(h, launch_cast_to_fp32(d, src[i], t[i]->dtype, (int) t[i]->fp_bias, t[i]->inf_nan_mode, i ? nb : na, 1.0f, 0, nullptr, 0, h->stream,
                                            flag, epoch));
     }
     g.dtype = DT_FP32;
@@ -554,10 +570,10 @@ int run_half_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor*
         g2.skip_epoch = epoch;
         g2.skip_if = 1;
         if (int rc = plan_launch(h, g2)) return rc; // (the workspace only grows: it now fits either request)
-        HIP_TRY(h, launch_gemm(g2, h->stream));
+        LAUNCH_TRY(h, launch_gemm(g2, h->stream));
     }
     if (int rc = plan_launch(h, g)) return rc;
-    HIP_TRY(h, launch_gemm(g, h->stream));
+    LAUNCH_TRY(h, launch_gemm(g, h->stream));
     return MME_HIP_OK;
 }
 
@@ -575,7 +591,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     if (int rc = plan_launch(h, g)) return rc;
     if (!is_fp8(g.dtype))
     {
-        HIP_TRY(h, launch_gemm(g, h->stream));
+        LAUNCH_TRY(h, launch_gemm(g, h->stream));
         return MME_HIP_OK;
     }
     const Fp8Plan plan = plan_fp8(ta, tb);
@@ -627,7 +643,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     }
     if (!need_scan)
     {
-        HIP_TRY(h, launch_gemm(g, h->stream));
+        LAUNCH_TRY(h, launch_gemm(g, h->stream));
         return MME_HIP_OK;
     }
     // the constants of the in-kernel look: a byte b is special when (b & m) == m, m = the exponent field (kind 0) or all of 0x7F
@@ -651,11 +667,11 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     {
         if (!h->chk_state.p) HIP_TRY(h, grow(h, h->chk_state, (size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS * sizeof(uint32_t)));
         const unsigned slot = h->chk_state_launches++ % CHK_STATE_RING;
-        if (slot == 0) HIP_TRY(h, launch_fill_u32((uint32_t*) h->chk_state.p, 0u, (size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS, h->stream));
+        if (slot == 0) LAUNCH_TRY(h, launch_fill_u32((uint32_t*) h->chk_state.p, 0u, (size_t) CHK_STATE_RING * CHK_STATE_REGION_WORDS, h->stream));
         g.chk = 2;
         g.chk_state = (uint32_t*) h->chk_state.p + (size_t) slot * CHK_STATE_REGION_WORDS;
         set_check_constants();
-        HIP_TRY(h, launch_gemm(g, h->stream));
+        LAUNCH_TRY(h, launch_gemm(g, h->stream));
         return MME_HIP_OK;
     }
     // the flag holds the epoch of the latest call that met such a code; the native kernel either finds them itself while it
@@ -673,9 +689,9 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
         set_check_constants();
     }
     else
-        HIP_TRY(h, launch_fp8_special_scan2(flag, epoch, a_base, span_elements(ta), ta->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[0], b_base,
+        LAUNCH_TRY(h, launch_fp8_special_scan2(flag, epoch, a_base, span_elements(ta), ta->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[0], b_base,
                                             span_elements(tb), tb->dtype == MME_HIP_FP8_143 ? 3 : 2, plan.scan_kind[1], h->stream));
-    HIP_TRY(h, launch_gemm(g, h->stream));
+    LAUNCH_TRY(h, launch_gemm(g, h->stream));
 
     const size_t na = span_elements(ta), nb = span_elements(tb);
     const size_t na_pad = (na + 7) & ~(size_t) 7;
@@ -683,7 +699,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     if (int rc = take_ws(h, h->decode_ws, (na_pad + nb + 8) * 2, &decode_ws)) return rc;
     uint16_t* da = (uint16_t*) decode_ws;
     uint16_t* db = da + na_pad;
-    HIP_TRY(h, launch_fp8_to_bf16_2(da, (const uint8_t*) a_base, na, ta->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) ta->fp_bias, ta->inf_nan_mode, db,
+    LAUNCH_TRY(h, launch_fp8_to_bf16_2(da, (const uint8_t*) a_base, na, ta->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) ta->fp_bias, ta->inf_nan_mode, db,
                                     (const uint8_t*) b_base, nb, tb->dtype == MME_HIP_FP8_143 ? 3 : 2, (int) tb->fp_bias, tb->inf_nan_mode, flag,
                                     epoch, h->stream));
     GemmProblem g2 = g;
@@ -705,7 +721,7 @@ int run_contraction(mme_hip_handle h, GemmProblem& g, const mme_hip_tensor* ta, 
     }
     g2.skip_if = 0; // decoded variant: skipped unless the scan found something
     g2.split_k = g.split_k;
-    HIP_TRY(h, launch_gemm(g2, h->stream));
+    LAUNCH_TRY(h, launch_gemm(g2, h->stream));
     return MME_HIP_OK;
 }
 
@@ -766,7 +782,7 @@ int with_stochastic_epilogue(mme_hip_handle h, const mme_hip_tensor* out, const 
     tmp.data = p;
     // gaps between strided rows are converted too (the cast runs over the tensor's span): they hold zeros, as a freshly
     // allocated accumulator tensor of the reference would
-    if (n != n_elements(out)) HIP_TRY(h, launch_fill_u32((uint32_t*) p, 0u, n, h->stream));
+    if (n != n_elements(out)) LAUNCH_TRY(h, launch_fill_u32((uint32_t*) p, 0u, n, h->stream));
     mme_hip_epilogue plain = *epi;
     plain.rounding_mode = MME_HIP_RM_NEAREST_EVEN;
     plain.clip_fp = plain.clip_inf_in = plain.flush_denorms = 0;
@@ -931,7 +947,7 @@ int mme_hip_clock_probe(mme_hip_handle h, int enable)
     const size_t bytes = (size_t) CLOCK_PROBE_WORKGROUPS * 4 * sizeof(uint64_t);
     HIP_TRY(h, hipSetDevice(h->device));
     HIP_TRY(h, grow(h, h->clock_probe_buf, bytes));
-    HIP_TRY(h, launch_fill_u32((uint32_t*) h->clock_probe_buf.p, 0, bytes / 4, h->stream));
+    LAUNCH_TRY(h, launch_fill_u32((uint32_t*) h->clock_probe_buf.p, 0, bytes / 4, h->stream));
     h->clock_probe = (uint64_t*) h->clock_probe_buf.p;
     return MME_HIP_OK;
 }
@@ -944,7 +960,7 @@ int mme_hip_clock_probe_read(mme_hip_handle h, double* shader_mhz, double* mean_
     std::vector<uint64_t> host(cells);
     HIP_TRY(h, hipSetDevice(h->device));
     HIP_TRY(h, hipMemcpyAsync(host.data(), h->clock_probe, cells * sizeof(uint64_t), hipMemcpyDeviceToHost, h->stream));
-    HIP_TRY(h, launch_fill_u32((uint32_t*) h->clock_probe, 0, cells * 2, h->stream));
+    LAUNCH_TRY(h, launch_fill_u32((uint32_t*) h->clock_probe, 0, cells * 2, h->stream));
     HIP_TRY(h, hipStreamSynchronize(h->stream));
     double clocks = 0, ticks = 0, worst = 0;
     int    n = 0;
@@ -1054,7 +1070,7 @@ int mme_hip_batch_gemm_dev(mme_hip_handle h, const mme_hip_tensor* out, const mm
         if (n_elements(x) != n_elements(w)) return fail(h, MME_HIP_EINVAL, "One of the input tensors is zero-size, while the other is not");
         const size_t bytes = span_elements(out) * out_es;
         if (bytes % 4) return fail(h, MME_HIP_EUNSUPPORTED, "zero-size contraction into an output whose byte size is not a multiple of 4");
-        HIP_TRY(h, launch_fill_u32((uint32_t*) out->data, 0u, bytes / 4, h->stream));
+        LAUNCH_TRY(h, launch_fill_u32((uint32_t*) out->data, 0u, bytes / 4, h->stream));
         return MME_HIP_OK;
     }
     const bool ta = (op == MME_HIP_OP_ATB || op == MME_HIP_OP_ATBT);
@@ -1145,11 +1161,11 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
                 a.sizes[i] = w->sizes[i], a.src_strides[i] = w->strides[i], a.dst_strides[i] = run;
                 run *= w->sizes[i];
             }
-            HIP_TRY(h, launch_strided_copy(ws, w->data, es, a, h->stream));
+            LAUNCH_TRY(h, launch_strided_copy(ws, w->data, es, a, h->stream));
             w_dense = ws;
         }
         if (int rc = take_ws(h, h->weights_ws, (size_t) acc * es + 16, &ws)) return rc;
-        HIP_TRY(h, launch_repack_transposed_weights(ws, w_dense, es, w->sizes[0], w->sizes[1], w->sizes[2], (size_t) acc, h->stream));
+        LAUNCH_TRY(h, launch_repack_transposed_weights(ws, w_dense, es, w->sizes[0], w->sizes[1], w->sizes[2], (size_t) acc, h->stream));
         mme_hip_tensor wr = *w;
         wr.data = ws;
         wr.sizes[0] = w->sizes[1];
@@ -1225,13 +1241,13 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
             {
                 if (int rc = take_ws(h, h->pack_ws[0], (size_t) n_elements(w) * elem_size(w->dtype) + 16, &p)) return rc;
                 wd = dense_of(w, p);
-                HIP_TRY(h, copy(&wd, w));
+                LAUNCH_TRY(h, copy(&wd, w));
             }
             if (pack_y)
             {
                 if (int rc = take_ws(h, h->pack_ws[1], (size_t) n_elements(y) * elem_size(y->dtype) + 16, &p)) return rc;
                 yd = dense_of(y, p);
-                HIP_TRY(h, copy(&yd, y));
+                LAUNCH_TRY(h, copy(&yd, y));
             }
             if (pack_out)
             {
@@ -1243,7 +1259,7 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
             const mme_hip_tensor* w2 = op == MME_HIP_OP_DEDW ? o2 : (pack_w ? &wd : w);
             const mme_hip_tensor* y2 = op == MME_HIP_OP_FWD ? o2 : (pack_y ? &yd : y);
             if (int rc = mme_hip_convolution_dev(h, o2, x2, w2, y2, cp, op, epi)) return rc;
-            if (pack_out) HIP_TRY(h, copy(out, &od));
+            if (pack_out) LAUNCH_TRY(h, copy(out, &od));
             return MME_HIP_OK;
         }
     }
@@ -1275,7 +1291,8 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
             GemmEpilogue e;
             if (int rc = fill_epilogue(h, e, out, epi)) return rc;
             e.ld = Kc;
-            HIP_TRY(h, launch_conv_fwd_fast(x->data, w->data, x->sizes[4], x->sizes[2], x->sizes[1], e, h->num_cus, h->status_dev, h->wait_limit, h->stream));
+            h->last_form[0] = 2, h->last_form[1] = 0, h->last_form[2] = 1, h->last_form[3] = 8; // (the 3 x 3, 64 -> 64 channel forward kernel)
+            LAUNCH_TRY(h, launch_conv_fwd_fast(x->data, w->data, x->sizes[4], x->sizes[2], x->sizes[1], e, h->num_cus, h->status_dev, h->wait_limit, h->stream));
             return MME_HIP_OK;
         }
     }
@@ -1351,6 +1368,51 @@ int mme_hip_convolution_dev(mme_hip_handle h, const mme_hip_tensor* out, const m
 
 namespace
 {
+// a handle for planning only: no device, no stream, nothing allocated; the registers and the jump table that a stochastic
+// epilogue's host bookkeeping reads are there (all zero)
+void make_planning_handle(mme_hip_calc& h, int num_cus, int fp8_specials_policy)
+{
+    h.dry_run = true;
+    h.num_cus = num_cus > 0 ? num_cus : 256;
+    h.fp8_specials_policy = fp8_specials_policy;
+    h.lfsr.assign(256, 0u);
+    h.lfsr_jump.assign((size_t) LFSR_JUMP_LEVELS * 32, 0u);
+}
+
+int planned_form(mme_hip_calc& h, int rc, int form[4], char* error, size_t error_bytes)
+{
+    for (int i = 0; i < 4; i++) form[i] = rc == MME_HIP_OK ? h.last_form[i] : 0;
+    if (error && error_bytes)
+    {
+        snprintf(error, error_bytes, "%s", rc == MME_HIP_OK ? "" : h.error.c_str());
+    }
+    return rc;
+}
+} // namespace
+
+int mme_hip_plan_batch_gemm(const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, int op, const mme_hip_epilogue* epi,
+                            int num_cus, int fp8_specials_policy, int form[4], char* error, size_t error_bytes)
+{
+    if (!form) return MME_HIP_EINVAL;
+    mme_hip_calc h;
+    make_planning_handle(h, num_cus, fp8_specials_policy);
+    h.last_form[0] = -1; // (a zero-size contraction launches no contraction kernel at all)
+    return planned_form(h, mme_hip_batch_gemm_dev(&h, out, x, w, op, epi), form, error, error_bytes);
+}
+
+int mme_hip_plan_convolution(const mme_hip_tensor* out, const mme_hip_tensor* x, const mme_hip_tensor* w, const mme_hip_tensor* y,
+                             const mme_hip_conv_params* cp, int op, const mme_hip_epilogue* epi, int num_cus, int fp8_specials_policy, int form[4],
+                             char* error, size_t error_bytes)
+{
+    if (!form) return MME_HIP_EINVAL;
+    mme_hip_calc h;
+    make_planning_handle(h, num_cus, fp8_specials_policy);
+    h.last_form[0] = -1;
+    return planned_form(h, mme_hip_convolution_dev(&h, out, x, w, y, cp, op, epi), form, error, error_bytes);
+}
+
+namespace
+{
 // jump table of the handle's LFSR: entry [k][b] = state reached from the one-bit state 1 << b after 2^k steps (built once, when
 // the calculator is created)
 int build_lfsr_jump(mme_hip_handle h)
@@ -1414,7 +1476,7 @@ int mme_hip_activation_dev(mme_hip_handle h, const mme_hip_tensor* out, const mm
         bool contiguous = acc->strides[0] == 1;
         for (int d = 1; d < acc->dim && d < MME_HIP_MAX_TENSOR_DIMS; d++) contiguous = contiguous && acc->strides[d] == acc->strides[d - 1] * acc->sizes[d - 1];
         if (!contiguous) return fail(h, MME_HIP_EINVAL, "input and output should be flattened");
-        HIP_TRY(h, launch_relu_inplace((float*) acc->data, n, h->stream));
+        LAUNCH_TRY(h, launch_relu_inplace((float*) acc->data, n, h->stream));
     }
     const CastParams c = make_cast(out->dtype, out->fp_bias, out->inf_nan_mode, rm, clip_fp, clip_inf_in, flush_denorms, 0, 0);
     const bool       reseed = rm == MME_HIP_RM_STOCHASTIC || rm == MME_HIP_RM_STOCHASTIC_AND_NEAREST || stochastic_ftz;
@@ -1427,12 +1489,12 @@ int mme_hip_activation_dev(mme_hip_handle h, const mme_hip_tensor* out, const mm
         LfsrRegisters regs;
         memset(&regs, 0, sizeof regs);
         for (size_t r = 0; r < L; r++) regs.v[r] = h->lfsr[r];
-        HIP_TRY(h, launch_cast_stochastic(out->data, (const float*) acc->data, n, c, stochastic_ftz, 1, h->polynomial, regs,
+        LAUNCH_TRY(h, launch_cast_stochastic(out->data, (const float*) acc->data, n, c, stochastic_ftz, 1, h->polynomial, regs,
                                           (const uint32_t*) h->lfsr_jump_dev.p, h->stream));
         for (size_t r = 0; r < L && r < n; r++) h->lfsr[r] = lfsr_jump_host(h, h->lfsr[r], (n - r + L - 1) / L);
         return MME_HIP_OK;
     }
-    HIP_TRY(h, launch_cast_from_fp32(out->data, (const float*) acc->data, n, c, nullptr, 0, h->stream));
+    LAUNCH_TRY(h, launch_cast_from_fp32(out->data, (const float*) acc->data, n, c, nullptr, 0, h->stream));
     return MME_HIP_OK;
 }
 
@@ -1449,7 +1511,7 @@ int mme_hip_cast_from_fp32_dev(mme_hip_handle h, void* out, int out_dtype, unsig
     if (col_scale_exp && n_cols == 0) return fail(h, MME_HIP_EINVAL, "n_cols must be positive with per-column scales");
     if (n && (!out || !in)) return fail(h, MME_HIP_EINVAL, "got null pointer");
     const CastParams c = make_cast(out_dtype, out_fp_bias, out_inf_nan_mode, rm, clip_fp, clip_inf_in, flush_denorms, relu, scale_exp);
-    HIP_TRY(h, launch_cast_from_fp32(out, in, n, c, col_scale_exp, n_cols, h->stream));
+    LAUNCH_TRY(h, launch_cast_from_fp32(out, in, n, c, col_scale_exp, n_cols, h->stream));
     return MME_HIP_OK;
 }
 
@@ -1461,7 +1523,7 @@ int mme_hip_cast_to_fp32_dev(mme_hip_handle h, float* out, const void* in, int i
     if (scale_exp < -126 || scale_exp > 126) return fail(h, MME_HIP_EINVAL, "scale exponent out of range");
     if (col_scale_exp && n_cols == 0) return fail(h, MME_HIP_EINVAL, "n_cols must be positive with per-column scales");
     if (n && (!out || !in)) return fail(h, MME_HIP_EINVAL, "got null pointer");
-    HIP_TRY(h, launch_cast_to_fp32(out, in, in_dtype, (int) in_fp_bias, in_inf_nan_mode, n, pow2f(scale_exp), scale_exp != 0, col_scale_exp,
+    LAUNCH_TRY(h, launch_cast_to_fp32(out, in, in_dtype, (int) in_fp_bias, in_inf_nan_mode, n, pow2f(scale_exp), scale_exp != 0, col_scale_exp,
                                    n_cols, h->stream));
     return MME_HIP_OK;
 }
@@ -1470,7 +1532,7 @@ int mme_hip_absmax_dev(mme_hip_handle h, float* out_absmax, const float* in, siz
 {
     if (!h) return MME_HIP_EINVAL;
     if (!out_absmax || (n && !in)) return fail(h, MME_HIP_EINVAL, "got null pointer");
-    HIP_TRY(h, launch_absmax(out_absmax, in, n, h->stream));
+    LAUNCH_TRY(h, launch_absmax(out_absmax, in, n, h->stream));
     return MME_HIP_OK;
 }
 
@@ -1695,7 +1757,7 @@ int mme_hip_memory_write_dev(mme_hip_handle h, const mme_hip_tensor* memory, con
     }
     if (mme_out->dtype != memory->dtype) return fail(h, MME_HIP_EINVAL, "element types of memory and mmeOut differ");
     if (reduction_rm < 0 || reduction_rm > 3) return fail(h, MME_HIP_EINVAL, "invalid reduction rounding mode %d", reduction_rm);
-    HIP_TRY(h, launch_memory_write_reduce(memory->data, mme_out->data, memory->dtype, n, reduction_op, reduction_rm,
+    LAUNCH_TRY(h, launch_memory_write_reduce(memory->data, mme_out->data, memory->dtype, n, reduction_op, reduction_rm,
                                           clip_fp, h->stream));
     return MME_HIP_OK;
 }

@@ -1,0 +1,108 @@
+"""The planner (mme_hip_plan_batch_gemm / mme_hip_plan_convolution): which kernel form a call would launch, answered by the
+library's own checking and planning code on a handle without a device.  No GPU needed.  Held to (a) the forms an MI355X
+reported after really launching every distinct contraction of the reference's Gaudi3 test configurations
+(tests/golden/contraction_forms.json, written by tests/golden/gen_contraction_forms.py) and (b) what the benchmark
+configurations are documented to take."""
+import json
+import os
+
+import pytest
+
+from intel_gaudi3_software_amd import abi, harness
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "contraction_forms.json")
+P = 4096  # stands in for a 16-byte aligned device address: the planner never dereferences it
+
+
+def T(sizes, dtype, bias=0, mode=0, strides=None):
+    return abi.make_tensor(P, sizes, dtype, bias, mode, strides, dim=5)
+
+
+def _plan_record(r):
+    a_l, b_l, o_l = {"dedx": ("y", "w", "x"), "transposed_dedx": ("y", "w", "x"), "dedw": ("x", "y", "w")}.get(r["op"], ("x", "w", "y"))
+    t = {"in_type": r["in_type"], "in2_type": r["in2_type"], "out_type": abi.FP32, "fp8_bias_in": 7 if r["in_type"] == abi.FP8_143 else 15,
+         "fp8_bias_in2": 7 if r["in2_type"] == abi.FP8_143 else 15, "fp8_bias_out": 0, "inf_nan_a": 0, "inf_nan_b": 0, "inf_nan_out": 0}
+    bias = {abi.FP8_143: 7, abi.FP8_152: 15, abi.FP16: 15, abi.UFP16: 31}
+    d = {a_l: T(r[a_l], r["in_type"], bias.get(r["in_type"], 0), 0, r[a_l + "_strides"]),
+         b_l: T(r[b_l], r["in2_type"], bias.get(r["in2_type"], 0), 0, r[b_l + "_strides"])}
+    acc = T(r[o_l], abi.FP32, 0, 0, r[o_l + "_strides"])
+    op = harness._OPS[r["op"]]
+    if op in harness._CONV_OPS:
+        cp = abi.make_conv_params(3, tuple(r["padding"]) + (0,), tuple(r["conv_strides"]) + (1,), tuple(r["dilation"]) + (1,))
+        return abi.plan_convolution(acc, d.get("x", acc), d.get("w", acc), d.get("y", acc), cp, op)
+    return abi.plan_batch_gemm(acc, d[a_l], d[b_l], op)
+
+
+def test_planner_reproduces_the_forms_the_gpu_reported():
+    rows = json.load(open(GOLDEN))
+    assert len(rows) == 197
+    large = 0
+    for r in rows:
+        got = _plan_record(r)
+        # (the 3 x 3 forward kernel reports its own form since the records were written; none of these cases takes it)
+        assert got["large_tile"] in (0, 1)
+        assert got == r["form"], (r["file"], r["op"], r["x"], r["w"], got, r["form"])
+        large += got["large_tile"] == 1
+    # what the record says about shapes that miss the large-tile kernels: 26 of 197 take one, 22 of the 81 with >= 0.2 GFLOP
+    assert large == 26
+    big = [r for r in rows if r["flops"] >= 2e8]
+    assert len(big) == 81 and sum(1 for r in big if r["form"]["large_tile"] == 1) == 22
+
+
+def test_planner_on_the_benchmark_configurations():
+    e = abi.Epilogue()
+    e.scale_exp, e.clip_fp = -10, 1
+    # fp8 4096^3 -> bf16: one round of 256 x 256 tiles, four wavefronts of 128 x 128
+    assert abi.plan_batch_gemm(T([4096, 4096], abi.BF16), T([4096, 4096], abi.FP8_143, 7), T([4096, 4096], abi.FP8_143, 7), abi.OP_AB, e) == \
+        {"large_tile": 1, "tile_rows": 256, "split_k": 1, "wavefronts": 4}
+    # ... a short reduction keeps eight wavefronts, and so does a shape with several rounds of tiles
+    assert abi.plan_batch_gemm(T([4096, 4096], abi.BF16), T([1024, 4096], abi.FP8_143, 7), T([4096, 1024], abi.FP8_143, 7), abi.OP_AB, e)["wavefronts"] == 8
+    assert abi.plan_batch_gemm(T([8192, 8192], abi.BF16), T([4096, 8192], abi.FP8_143, 7), T([8192, 4096], abi.FP8_143, 7), abi.OP_AB, e)["wavefronts"] == 8
+    # bf16 512^3: 128-row tiles (four 256-row tiles would use four compute units)
+    assert abi.plan_batch_gemm(T([512, 512], abi.FP32), T([512, 512], abi.BF16), T([512, 512], abi.BF16), abi.OP_AB) == \
+        {"large_tile": 1, "tile_rows": 128, "split_k": 1, "wavefronts": 8}
+    # the batched mixed-fp8 GEMM: 256-row tiles, no split (the persistent walk)
+    e5 = abi.Epilogue()
+    e5.scale_exp, e5.clip_fp, e5.col_scale_exp = 2, 1, P
+    assert abi.plan_batch_gemm(T([14336, 2048, 4], abi.FP8_143, 7), T([4096, 2048, 4], abi.FP8_143, 7), T([14336, 4096, 1], abi.FP8_152, 15), abi.OP_AB, e5) == \
+        {"large_tile": 1, "tile_rows": 256, "split_k": 1, "wavefronts": 8}
+    cp = abi.make_conv_params(2, (1, 1, 0), (1, 1, 1), (1, 1, 1))
+    xs, ws, ys = [256, 28, 28, 1, 32], [256, 256, 3, 3, 1], [256, 28, 28, 1, 32]
+    X, W, Y = T(xs, abi.BF16), T(ws, abi.BF16), T(ys, abi.BF16)
+    assert abi.plan_convolution(T(xs, abi.FP32), T(xs, abi.FP32), W, Y, cp, abi.OP_DEDX) == {"large_tile": 1, "tile_rows": 128, "split_k": 1, "wavefronts": 8}
+    assert abi.plan_convolution(T(ws, abi.FP32), X, T(ws, abi.FP32), Y, cp, abi.OP_DEDW) == {"large_tile": 1, "tile_rows": 128, "split_k": 14, "wavefronts": 8}
+    xs, ws, ys = [64, 56, 56, 1, 64], [64, 64, 3, 3, 1], [64, 56, 56, 1, 64]
+    ec = abi.Epilogue()
+    ec.clip_fp = 1
+    assert abi.plan_convolution(T(ys, abi.BF16), T(xs, abi.BF16), T(ws, abi.BF16), T(ys, abi.BF16), cp, abi.OP_FWD, ec)["large_tile"] == 2
+
+
+def test_planner_shows_the_cliff_of_one_odd_dimension():
+    """A reduction length that is not a multiple of 128 bytes, or rows that are not 16-byte aligned, leave the large-tile
+    kernels: the planner makes that visible without a GPU."""
+    ok = abi.plan_batch_gemm(T([4096, 4096], abi.FP32), T([4096, 4096], abi.BF16), T([4096, 4096], abi.BF16), abi.OP_AB)
+    assert ok["large_tile"] == 1
+    for k in (4100, 4104, 4128):
+        odd = abi.plan_batch_gemm(T([4096, 4096], abi.FP32), T([k, 4096], abi.BF16), T([4096, k], abi.BF16), abi.OP_AB)
+        assert odd["large_tile"] == 0, k
+    assert abi.plan_batch_gemm(T([4096, 4096], abi.FP32), T([4160, 4096], abi.BF16), T([4096, 4160], abi.BF16), abi.OP_AB)["large_tile"] == 1
+    # partial tiles are taken (N a multiple of 16 from 128 columns, any M from 64 rows)
+    assert abi.plan_batch_gemm(T([4000, 3000], abi.FP32), T([4096, 3000], abi.BF16), T([4000, 4096], abi.BF16), abi.OP_AB)["large_tile"] == 1
+    assert abi.plan_batch_gemm(T([4001, 3000], abi.FP32), T([4096, 3000], abi.BF16), T([4001, 4096], abi.BF16), abi.OP_AB)["large_tile"] == 0
+
+
+def test_planner_refuses_what_the_calculator_refuses():
+    with pytest.raises(ValueError, match="Common dim"):
+        abi.plan_batch_gemm(T([512, 512], abi.FP32), T([512, 512], abi.BF16), T([512, 500], abi.BF16), abi.OP_AB)
+    with pytest.raises(ValueError, match="mixed input type"):
+        abi.plan_batch_gemm(T([512, 512], abi.FP32), T([512, 512], abi.BF16), T([512, 512], abi.FP32), abi.OP_AB)
+    # a zero-size common dimension launches no contraction kernel
+    assert abi.plan_batch_gemm(T([8, 8], abi.FP32), T([0, 8], abi.BF16), T([8, 0], abi.BF16), abi.OP_AB)["large_tile"] == -1
+    # the fp8 policy is part of the plan's input (it does not change the form, only what rides along)
+    a = abi.plan_batch_gemm(T([4096, 4096], abi.FP32), T([4096, 4096], abi.FP8_143, 7), T([4096, 4096], abi.FP8_143, 7), abi.OP_AB,
+                            fp8_specials_policy=abi.FP8_SPECIALS_ASSUME_NONE)
+    assert a["large_tile"] == 1 and a["wavefronts"] == 4
+    # a stochastic epilogue plans through the fp32 intermediate
+    e = abi.Epilogue()
+    e.rounding_mode = 4
+    assert abi.plan_batch_gemm(T([512, 512], abi.BF16), T([512, 512], abi.BF16), T([512, 512], abi.BF16), abi.OP_AB, e)["large_tile"] == 1
