@@ -265,6 +265,40 @@ public:
     void  setOperandClip(bool clipFp, bool clipFpInfIn) { check(mme_hip_set_operand_clip(m_h, clipFp, clipFpInfIn)); }
     mme_hip_handle handle() const { return m_h; }
 
+    /* Which kernel form a device-resident call would launch, without making it and without a device (mme_hip_plan_batch_gemm /
+     * mme_hip_plan_convolution; no counterpart in the reference): the descriptors go through the same checks and planning as
+     * the real call, their data pointers are not dereferenced.  Throws like the real call for a problem it would refuse. */
+    struct Form
+    {
+        int largeTile;  /* 1 a large-tile kernel, 0 the general kernel, 2 the 3 x 3 forward kernel, -1 no contraction kernel */
+        int tileRows;   /* 256 or 128 */
+        int splitK;     /* slices of the reduction, 1: none */
+        int wavefronts; /* per workgroup: 8 or 4 */
+    };
+    template<class T>
+    static Form planBatchGemm(const T& outputTensor, const T& xTensor, const T& wTensor, int op, const Epilogue* epilogue = nullptr, int numCus = 256,
+                              int fp8SpecialsPolicy = MME_HIP_FP8_SPECIALS_CHECK)
+    {
+        const mme_hip_tensor o = pod(outputTensor), x = pod(xTensor), w = pod(wTensor);
+        int                  form[4];
+        char                 error[512];
+        const int            rc = mme_hip_plan_batch_gemm(&o, &x, &w, op, epilogue, numCus, fp8SpecialsPolicy, form, error, sizeof error);
+        if (rc != MME_HIP_OK) throw MMEStackException(error, rc);
+        return Form {form[0], form[1], form[2], form[3]};
+    }
+    template<class T, class P>
+    static Form planConvolution(const T& outputTensor, const T& xTensor, const T& wTensor, const T& yTensor, const P& params, int op,
+                                const Epilogue* epilogue = nullptr, int numCus = 256, int fp8SpecialsPolicy = MME_HIP_FP8_SPECIALS_CHECK)
+    {
+        const mme_hip_tensor      o = pod(outputTensor), x = pod(xTensor), w = pod(wTensor), y = pod(yTensor);
+        const mme_hip_conv_params p = pod_conv(params);
+        int                       form[4];
+        char                      error[512];
+        const int rc = mme_hip_plan_convolution(&o, &x, &w, &y, &p, op, epilogue, numCus, fp8SpecialsPolicy, form, error, sizeof error);
+        if (rc != MME_HIP_OK) throw MMEStackException(error, rc);
+        return Form {form[0], form[1], form[2], form[3]};
+    }
+
 private:
     template<class T>
     static mme_hip_tensor pod(const T& t)

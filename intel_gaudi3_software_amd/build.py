@@ -54,14 +54,18 @@ def build_library(verbose=False, jobs=8, only_changed=False):
 
 
 def build_cpp_tests():
-    """Compile the C++ known-answer program of the calculator header (host code only, g++)."""
+    """Compile the C++ programs over the calculator header (host code only, g++): the known-answer program (needs a GPU to
+    run) and the planner's (runs anywhere).  Returns the path of the first."""
     root = os.path.dirname(_HERE)
-    src = os.path.join(root, "tests", "cpp", "kat_calculator.cpp")
-    exe = os.path.join(root, "tests", "cpp", "kat_calculator")
-    cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(root, "include"), src, "-o", exe, "-L" + CSRC,
-           "-lmme_hip", "-Wl,-rpath,$ORIGIN/../../intel_gaudi3_software_amd/csrc"]
-    subprocess.check_call(cmd)
-    return exe
+    exes = []
+    for name in ("kat_calculator", "plan_calculator"):
+        src = os.path.join(root, "tests", "cpp", name + ".cpp")
+        exe = os.path.join(root, "tests", "cpp", name)
+        cmd = [os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(root, "include"), src, "-o", exe, "-L" + CSRC,
+               "-lmme_hip", "-Wl,-rpath,$ORIGIN/../../intel_gaudi3_software_amd/csrc"]
+        subprocess.check_call(cmd)
+        exes.append(exe)
+    return exes[0]
 
 
 def _resource_report(text):

@@ -106,3 +106,19 @@ def test_planner_refuses_what_the_calculator_refuses():
     e = abi.Epilogue()
     e.rounding_mode = 4
     assert abi.plan_batch_gemm(T([512, 512], abi.BF16), T([512, 512], abi.BF16), T([512, 512], abi.BF16), abi.OP_AB, e)["large_tile"] == 1
+
+
+def test_planner_through_the_cpp_header():
+    """MmeHip::Calculator::planBatchGemm / planConvolution (include/mme_hip_calculator.h) in tests/cpp/plan_calculator.cpp, built
+    by intel_gaudi3_software_amd.build.build_cpp_tests() and run as a child process; no GPU."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "cpp", "plan_calculator")
+    if not os.path.exists(exe):  # (host code only: g++ over the header, two seconds)
+        from intel_gaudi3_software_amd import build
+        build.build_cpp_tests()
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=60)
+    text = r.stdout.decode(errors="replace")
+    print(text)
+    assert r.returncode == 0, text
+    assert text.count("ok    ") == 4 and "all ok" in text and "FAILED" not in text
