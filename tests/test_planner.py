@@ -122,3 +122,111 @@ def test_planner_through_the_cpp_header():
     print(text)
     assert r.returncode == 0, text
     assert text.count("ok    ") == 4 and "all ok" in text and "FAILED" not in text
+
+
+def test_planned_forms_respect_what_the_kernels_assume():
+    """The large-tile kernels count on whole 64-byte stages in even numbers, at least six per k-slice, operand rows that are
+    multiples of 16 bytes and outputs in groups of 16 columns; the four-wavefront form on fp8 operands, whole 256-row tiles in
+    one round and a long reduction.  Whatever the planner picks for a few thousand shapes around the boundaries must stay
+    inside those assumptions (a plan outside them would be a launch that reads or writes out of bounds)."""
+    import numpy as np
+    rng = np.random.default_rng(2024)
+    es_of = {abi.BF16: 2, abi.FP16: 2, abi.FP8_143: 1, abi.FP8_152: 1}
+    seen_split = seen_w4 = seen_128 = seen_large = 0
+    for trial in range(4000):
+        dt = [abi.BF16, abi.FP16, abi.FP8_143, abi.FP8_152][int(rng.integers(4))]
+        es = es_of[dt]
+        bias = {abi.FP8_143: 7, abi.FP8_152: 15, abi.FP16: 15}.get(dt, 0)
+        pick = lambda unit, hi: int(rng.integers(1, hi)) * unit + (int(rng.integers(0, unit)) if rng.random() < 0.2 else 0)
+        M, N, K = pick(64, 80), pick(64, 80), pick(64, 160)
+        nb = int(rng.choice([1, 1, 1, 2, 5]))
+        op = int(rng.choice([abi.OP_AB, abi.OP_ABT, abi.OP_ATB, abi.OP_ATBT]))
+        if trial % 10 == 0:
+            # the neighbourhood of the four-wavefront form: fp8, whole 256-row tiles around one round, long reductions
+            dt, es, bias = abi.FP8_143, 1, 7
+            M, N, K, nb = 256 * int(rng.integers(4, 20)), 256 * int(rng.integers(4, 20)), 128 * int(rng.integers(16, 40)), int(rng.choice([1, 1, 2]))
+            op = int(rng.choice([abi.OP_AB, abi.OP_ABT]))
+        ta, tb = op in (abi.OP_ATB, abi.OP_ATBT), op in (abi.OP_ABT, abi.OP_ATBT)
+        x = T([M, K, nb] if ta else [K, M, nb], dt, bias)
+        w = T([K, N, nb] if tb else [N, K, nb], dt, bias)
+        f = abi.plan_batch_gemm(T([N, M, nb], abi.FP32), x, w, op, num_cus=256, fp8_specials_policy=int(rng.integers(2)))
+        if f["large_tile"] != 1:
+            continue
+        seen_large += 1
+        kb = K * es
+        assert kb % 128 == 0 and kb >= 384, (M, N, K, dt, f)
+        assert N % 16 == 0 and N >= 128 and M >= 64, (M, N, K, dt, f)
+        # operand rows in multiples of 16 bytes
+        assert ((M if ta else K) * es) % 16 == 0 and ((K if tb else N) * es) % 16 == 0, (M, N, K, op, dt, f)
+        assert f["tile_rows"] in (128, 256) and f["wavefronts"] in (4, 8) and f["split_k"] >= 1
+        nk = kb // 64
+        if f["split_k"] > 1:
+            seen_split += 1
+            assert nk % (2 * f["split_k"]) == 0 and nk // f["split_k"] >= 6, (M, N, K, dt, f)
+        if f["tile_rows"] == 128:
+            seen_128 += 1
+        if f["wavefronts"] == 4:
+            seen_w4 += 1
+            tiles = (M // 256) * (N // 256) * nb
+            assert es == 1 and not ta and M % 256 == 0 and N % 256 == 0 and f["tile_rows"] == 256 and f["split_k"] == 1 and tiles <= 256 and nk >= 48, (M, N, K, f)
+        if ta and (M % 256 or N % 256):
+            # A contiguous along the tile's rows has no partial-tile kernels (the 2-byte types: whole 128- or 256-row tiles)
+            assert es == 2 and M % 128 == 0 and N % 256 == 0, (M, N, K, op, f)
+    assert seen_large > 500 and seen_split > 20 and seen_128 > 20 and seen_w4 > 5, (seen_large, seen_split, seen_128, seen_w4)
+
+
+def test_planned_convolution_forms_respect_what_the_gather_kernels_assume():
+    """The same for convolutions: the gather of fwd / dedx stages whole 64-byte runs of channels inside one filter tap (at most 32
+    taps), dedw 16-byte runs; dedx in gather form exists for unit convolution strides only; the weights' channel extents are
+    16-byte multiples; k-slices hold an even number of stages, at least six."""
+    import numpy as np
+    rng = np.random.default_rng(77)
+    large = {abi.OP_FWD: 0, abi.OP_DEDX: 0, abi.OP_DEDW: 0}
+    split = 0
+    for trial in range(3000):
+        dt = [abi.BF16, abi.FP16, abi.FP8_143][int(rng.integers(3))]
+        es = 1 if dt == abi.FP8_143 else 2
+        bias = {abi.FP8_143: 7, abi.FP16: 15}.get(dt, 0)
+        C = int(rng.choice([8, 16, 24, 32, 48, 64, 96, 128, 200, 256, 320]))
+        Kc = int(rng.choice([16, 64, 100, 128, 192, 256, 320, 512]))
+        S, R, Q = int(rng.integers(1, 4)), int(rng.integers(1, 4)), int(rng.choice([1, 1, 1, 2, 4]))
+        W, H, D, B = int(rng.integers(6, 40)), int(rng.integers(6, 40)), int(rng.choice([1, 1, 3])), int(rng.integers(1, 9))
+        st = [int(rng.choice([1, 1, 1, 2])) for _ in range(3)]
+        di = [int(rng.choice([1, 1, 1, 2])) for _ in range(3)]
+        pad = [int(rng.integers(0, 2)) for _ in range(3)]
+        if D == 1:
+            Q, st[2], di[2], pad[2] = 1, 1, 1, 0
+        out = [(n + 2 * p - d * (k - 1) - 1) // s + 1 for n, p, d, k, s in zip((W, H, D), pad, di, (S, R, Q), st)]
+        if min(out) < 1:
+            continue
+        xs, ws, ys = [C, W, H, D, B], [Kc, C, S, R, Q], [Kc, out[0], out[1], out[2], B]
+        cp = abi.make_conv_params(3, tuple(pad) + (0,), tuple(st) + (1,), tuple(di) + (1,))
+        op = [abi.OP_FWD, abi.OP_DEDX, abi.OP_DEDW][int(rng.integers(3))]
+        X, Wt, Y = T(xs, dt, bias), T(ws, dt, bias), T(ys, dt, bias)
+        if op == abi.OP_FWD:
+            f = abi.plan_convolution(T(ys, abi.FP32), X, Wt, T(ys, abi.FP32), cp, op)
+        elif op == abi.OP_DEDX:
+            f = abi.plan_convolution(T(xs, abi.FP32), T(xs, abi.FP32), Wt, Y, cp, op)
+        else:
+            f = abi.plan_convolution(T(ws, abi.FP32), X, T(ws, abi.FP32), Y, cp, op)
+        if f["large_tile"] != 1:
+            continue
+        large[op] += 1
+        taps = S * R * Q
+        assert taps <= 32, (xs, ws, f)
+        nch, n_out = (C, Kc) if op == abi.OP_FWD else ((Kc, C) if op == abi.OP_DEDX else (C, Kc))
+        assert n_out % 16 == 0 and n_out >= 128, (op, xs, ws, f)
+        if op == abi.OP_DEDW:
+            assert (nch * es) % 16 == 0, (xs, ws, f)
+            kb = B * out[0] * out[1] * out[2] * es   # the reduction runs over the output pixels
+        else:
+            assert (nch * es) % 64 == 0, (op, xs, ws, f)
+            kb = taps * nch * es
+        if op == abi.OP_DEDX:
+            assert st == [1, 1, 1], (xs, ws, st, f)
+        assert kb % 128 == 0 and kb >= 384, (op, xs, ws, ys, f)
+        if f["split_k"] > 1:
+            split += 1
+            nk = kb // 64
+            assert nk % (2 * f["split_k"]) == 0 and nk // f["split_k"] >= 6, (op, xs, ws, f)
+    assert min(large.values()) > 20 and split > 10, (large, split)
